@@ -491,6 +491,62 @@ int tm_gemm_export(const char* path);
 
 
 /* ----------------------------------------------------------------------------------------------
+ * Layer-list models: a decoder described layer by layer (mixer kind, the mixer's sizes and constants, feed-forward), fp32 residual
+ * stream, unquantised bf16 weights.  Runs on the same engine: block pool, scheduler, static batch, continuous batching, sampling.
+ *   block:  x <- x + residual_mult * (mixer(norm1(x)) + ff(norm2(x))), both norms of the same x (ff absent: mlp = TM_MLP_NONE)
+ *   norm:   x / sqrt(mean(x^2) + norm_eps) * (norm_offset + w)
+ *   mixer TM_MIXER_ATTENTION: grouped-query causal attention without rotation, key size dim, value size vdim,
+ *           score = cap(q . k * scale * (1 + qtemp_coef * ln(floor((p + 1) / qtemp_every) + 1))), cap(s) = softcap * tanh(s / softcap)
+ *           (softcap <= 0: none; qtemp_coef = 0: none), soft-max whose denominator holds exp(sink[head]) when sink != 0
+ *   ff TM_MLP_DENSE: down(act(up(h))), act = TM_ACT_RELU2: relu(z)^2
+ *   logits = head(norm(x)) * logit_scale
+ * weights_of >= 0: the layer has no tensors, it runs on that layer's (which must own its tensors) with a cache of its own.
+ * dtype: TM_DTYPE_BF16 -- matrix products and activations bf16 with fp32 accumulation, cache bf16; TM_DTYPE_F32 -- everything fp32.
+ * Norms, attention scores and weights, and the residual sum are fp32 in both.
+ * Weight slots (tm_engine_weight_copy, checkpoint bytes: bf16, [out][in]): "embed", "l<i>.norm1", "l<i>.norm2" (with an ff),
+ * "l<i>.mix.q|k|v|o", "l<i>.mix.sink" (with a sink), "l<i>.mlp.up|down", "final.norm", "head". */
+enum { TM_MIXER_ATTENTION = 1 };
+enum { TM_MLP_NONE = 0, TM_MLP_DENSE = 1 };
+enum { TM_ACT_RELU2 = 0 };
+enum { TM_DTYPE_BF16 = 0, TM_DTYPE_F32 = 1 };
+typedef struct tm_layer_spec {
+    int   mixer;
+    int   weights_of; /* -1: own tensors */
+    int   heads, kv_heads, dim, vdim;
+    float scale, softcap, qtemp_coef, qtemp_every;
+    int   sink;
+    int   mlp, ff, act;
+} tm_layer_spec;
+typedef struct tm_layered_config {
+    int                  width, vocab, n_layers;
+    const tm_layer_spec* layers;
+    float                norm_eps, norm_offset, residual_mult, logit_scale;
+    int                  dtype;
+} tm_layered_config;
+/* cfg->model is ignored; tp must be 1; quant_policy 0 (the cache holds the activation type) */
+int tm_engine_create_layered(tm_engine** out, const tm_engine_config* cfg, const tm_layered_config* model);
+
+/* Sessions: the caller feeds token ids and reads logits -- the forward, cache and scheduler bookkeeping of generation without the
+ * sampler (scoring, replaying recorded steps).  A session takes a batch slot of the scheduler; its cache blocks are taken from the
+ * pool as it grows and return when it closes.  tm_engine_step_tokens runs ONE forward over the next tokens of any set of open sessions
+ * (portions of prompts beside single tokens) and copies the fp32 logits of the wanted places (indices into an entry's tokens), in entry
+ * order, to host_logits [sum n_want][vocab].  TM_OOM: the pool cannot hold the step; TM_CONFLICT: queued / running requests exist
+ * (sessions and tm_engine_submit do not share a scheduler session).  Layer-list models only. */
+typedef struct tm_step_entry {
+    int64_t    session;
+    const int* tokens;
+    int        n_tokens;
+    const int* want;
+    int        n_want;
+} tm_step_entry;
+int tm_engine_session_open(tm_engine* e, int64_t* session);
+int tm_engine_session_close(tm_engine* e, int64_t session);
+int tm_engine_step_tokens(tm_engine* e, const tm_step_entry* entries, int n_entries, float* host_logits);
+/* parity tests (layer-list models): the next forwards stop behind `layers` layers (< 0: run all); the fp32 residual stream of the last
+ * forward is tm_engine_debug_read(what = 0) with bytes = rows * width * 4 */
+int tm_engine_debug_stop_after(tm_engine* e, int layers);
+
+/* ----------------------------------------------------------------------------------------------
  * Continuous batching.  Replaces ModelRequest.forward / cancel + the engine thread's
  * schedule-forward-update loop (bind.cpp:743-793, engine/engine.cc:434-470,770-870, model_request.cc:36-135):
  * requests are queued, admitted in arrival order when a batch slot and enough KV blocks (prompt + max_new_tokens,

@@ -67,6 +67,24 @@ class EngineConfig(C.Structure):
                 ('max_prefill_token_num', c_int), ('decode_splits', c_int), ('use_graph', c_int)]
 
 
+class LayerSpec(C.Structure):
+    """struct tm_layer_spec"""
+    _fields_ = [('mixer', c_int), ('weights_of', c_int), ('heads', c_int), ('kv_heads', c_int), ('dim', c_int), ('vdim', c_int),
+                ('scale', c_float), ('softcap', c_float), ('qtemp_coef', c_float), ('qtemp_every', c_float), ('sink', c_int),
+                ('mlp', c_int), ('ff', c_int), ('act', c_int)]
+
+
+class LayeredConfig(C.Structure):
+    """struct tm_layered_config"""
+    _fields_ = [('width', c_int), ('vocab', c_int), ('n_layers', c_int), ('layers', POINTER(LayerSpec)), ('norm_eps', c_float),
+                ('norm_offset', c_float), ('residual_mult', c_float), ('logit_scale', c_float), ('dtype', c_int)]
+
+
+class StepEntry(C.Structure):
+    """struct tm_step_entry"""
+    _fields_ = [('session', c_int64), ('tokens', c_void_p), ('n_tokens', c_int), ('want', c_void_p), ('n_want', c_int)]
+
+
 # name -> (restype, argtypes); every int-returning function is a tm_status
 _SIGNATURES = {
     'tm_version': (c_int, []),
@@ -157,6 +175,11 @@ _SIGNATURES = {
     'tm_p2p_allgather': (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     'tm_engine_create': (c_int, [POINTER(c_void_p), POINTER(EngineConfig)]),
     'tm_engine_destroy': (c_int, [c_void_p]),
+    'tm_engine_create_layered': (c_int, [POINTER(c_void_p), POINTER(EngineConfig), POINTER(LayeredConfig)]),
+    'tm_engine_session_open': (c_int, [c_void_p, POINTER(c_int64)]),
+    'tm_engine_session_close': (c_int, [c_void_p, c_int64]),
+    'tm_engine_step_tokens': (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
+    'tm_engine_debug_stop_after': (c_int, [c_void_p, c_int]),
     'tm_comm_unique_id': (c_int, [c_void_p]),
     'tm_engine_comm_init': (c_int, [c_void_p, c_void_p]),
     'tm_engine_weight_bytes': (c_int64, [c_void_p, c_char_p]),
@@ -228,10 +251,12 @@ def load():
     # Load order: PyTorch-ROCm bundles its own libamdhip64 / libhsa-runtime64; when this library (linked against
     # /opt/rocm) is loaded FIRST and torch later, the process ends up with mismatched runtimes and aborts at exit
     # ("double free or corruption").  torch first is the order every GPU test and bench run uses.
-    try:
-        import torch  # noqa: F401
-    except ImportError:
-        pass
+    # (TM_SKIP_TORCH_PRELOAD=1: a process that never imports torch -- a command-line tool -- skips the import and its start-up cost)
+    if not os.environ.get('TM_SKIP_TORCH_PRELOAD'):
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
     lib = C.CDLL(_LIB_PATH, mode=C.RTLD_GLOBAL)
     for name, (res, args) in _SIGNATURES.items():
         fn = getattr(lib, name)          # AttributeError if the .so does not export a declared symbol

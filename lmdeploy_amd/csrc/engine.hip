@@ -275,6 +275,9 @@ int tm_engine_init_synthetic(tm_engine* e, uint64_t seed)
 {
     TM_REQUIRE(e, "null pointer");
     TM_REQUIRE(!e->weights_ready, "weights already processed");
+    if (e->lm) {
+        return layered_init_synthetic(e, seed);
+    }
     const tm_model_config& m = e->cfg.model;
     uint64_t               sd = seed * 1000003ull + 17;
     half_t*                master = nullptr;  // fp16 master of the largest linear, reused
@@ -370,6 +373,9 @@ int tm_engine_process_weights(tm_engine* e)
         return 0;
     }
     TM_HIP_CHECK(hipSetDevice(e->cfg.device));
+    if (e->lm) {
+        return layered_process_weights(e);
+    }
     const tm_model_config& m = e->cfg.model;
     auto norm = [&](const std::string& name, half_t** dst) -> int {
         Slot& s = e->slots[name];
@@ -438,6 +444,9 @@ int tm_engine_start(tm_engine* e)
         return 0;
     }
     TM_HIP_CHECK(hipSetDevice(e->cfg.device));
+    if (e->lm) {
+        return layered_start(e);
+    }
     const tm_engine_config& c = e->cfg;
     const tm_model_config&  m = c.model;
     const int bits = c.quant_policy == 0 ? 16 : c.quant_policy;
@@ -606,6 +615,11 @@ int tm_engine_debug_read(tm_engine* e, int what, int a, int b, void* host_out, i
 {
     TM_REQUIRE(e && host_out && e->started, "null pointer / engine not started");
     TM_HIP_CHECK(hipStreamSynchronize(e->stream));
+    if (what == 0 && e->lm) {  // layer-list models keep the residual stream in fp32
+        TM_REQUIRE(a >= 1 && a <= e->max_tokens && bytes == (int64_t)a * e->hidden * 4, "residual rows / byte count");
+        TM_HIP_CHECK(hipMemcpy(host_out, e->lm->d_res, (size_t)bytes, hipMemcpyDeviceToHost));
+        return 0;
+    }
     if (what == 0) {  // residual stream of the last forward: rows [0, a)
         TM_REQUIRE(a >= 1 && a <= e->max_tokens && bytes == (int64_t)a * e->hidden * 2, "residual rows / byte count");
         TM_HIP_CHECK(hipMemcpy(host_out, e->d_resid, (size_t)bytes, hipMemcpyDeviceToHost));
@@ -653,6 +667,13 @@ int tm_engine_stats(tm_engine* e, int64_t* weight_bytes, int64_t* kv_bytes_per_t
         }
     }
     wb += (int64_t)e->output.w.packed_bytes;
+    if (e->lm) {
+        for (size_t i = 0; i < e->lm->layers.size(); ++i) {
+            const LmLayer& L = e->lm->layers[i];
+            wb += L.src == (int)i ? (int64_t)(L.qkv.bytes + L.up.bytes + L.out.bytes) : 0;
+        }
+        wb += (int64_t)e->lm->head.bytes;
+    }
     if (weight_bytes) *weight_bytes = wb;
     if (kv_bytes_per_token) *kv_bytes_per_token = e->started ? e->block_bytes / 64 : 0;
     if (num_blocks) *num_blocks = e->num_blocks;
@@ -719,6 +740,7 @@ int tm_engine_destroy(tm_engine* e)
         (void)hipFree(e->d_moe_ws);
     }
     linear_weight_free(e->output.w);
+    layered_free(e);
     for (auto& kv : e->slots) {
         if (kv.second.dev) {
             (void)hipFree(kv.second.dev);

@@ -341,6 +341,92 @@ static int linear_fold_produce(tm_engine* e, LinearSlots& l, const half_t* x, in
     return 0;
 }
 
+// Logits rows -> next ids for `n` sequences whose fp16 logits lie in d_logits at the batch slots [slot, slot + n): logits processors
+// (ids_in / cu_q (nullptr: one token per sequence) / ntok = the tokens this forward consumed for them, k_len = their context lengths),
+// then stochastic sampling or arg-max (tensor-parallel: over the gathered vocabulary shards).  Shared by every model family.
+int sample_rows(tm_engine* e, int n, int slot, const int* ids_in, const int* cu_q, int ntok, const int* k_len, const int* active)
+{
+    const tm_model_config& m      = e->cfg.model;
+    hipStream_t            st     = e->stream;
+    half_t*                logits = e->d_logits + (size_t)slot * e->vocab_local;
+    int*                   ids    = e->d_next_ids + slot;
+    if (e->logits_on) {
+        // the tokens this forward consumed join the slots' seen masks, then penalty / bans on the (local) logits
+        uint32_t* seen = e->d_seen + (size_t)slot * e->seen_words;
+        TM_PROF(P_SAMPLE, TM_TRY(launch_seen_update(seen, e->seen_words, ids_in, cu_q, n, ntok, m.vocab, st, active)));
+        TM_PROF(P_SAMPLE, TM_TRY(launch_logits_process(logits, n, e->vocab_local, e->vocab_local,
+                                                       e->vocab_local < m.vocab ? e->cfg.rank * e->vocab_local : 0, seen,
+                                                       e->seen_words, e->d_lp_rep + slot, e->d_lp_ban + slot * kMaxBadIds,
+                                                       e->d_lp_end + slot * kMaxEndIds, k_len, e->d_lp_minlen + slot, st)));
+    }
+    if (e->sampling_on && (!e->use_comm || ((e->comm || e->p2p_ready) && e->d_logits_full))) {
+        // parameters are indexed by batch slot, the counter (context length) by the row of this forward
+        const half_t* lg = logits;
+        int           V  = e->vocab_local;
+        if (e->use_comm) {
+            // tp > 1: the vocabulary shards are all-gathered into full rows (the reference gathers the logits too,
+            // models/language_model.cc:304-333) and EVERY rank draws from the same distribution with the same Philox
+            // number -> the same token everywhere, no further exchange
+            const size_t cnt = (size_t)n * e->vocab_local;
+            if (!e->comm) {
+                // native communicator alone: the shards travel through the P2P segments, as many whole rows per exchange as
+                // one segment buffer holds; rank q's rows land in its [n][vocab / tp] plane of d_logits_gather
+                half_t*   data[8];
+                uint32_t* flags[8];
+                p2p_tables(e, data, flags);
+                const size_t tile = (size_t)e->p2p_rows * e->hidden;  // fp16 elements of one segment buffer
+                const int    per  = (int)std::min<size_t>(n, tile / e->vocab_local);
+                TM_REQUIRE(per >= 1, "native communicator: one logits row does not fit a segment buffer (export more rows)");
+                for (int r0 = 0; r0 < n; r0 += per) {
+                    const int rows = std::min(per, n - r0);
+                    TM_TRY(launch_p2p_allgather(data, flags, e->cfg.tp, e->cfg.rank, e->p2p_state, tile, logits + (size_t)r0 * e->vocab_local,
+                                                e->d_logits_gather + (size_t)r0 * e->vocab_local, rows * e->vocab_local / 2, st,
+                                                cnt / 2));
+                }
+            }
+            else {
+                TM_NCCL_CHECK(ncclAllGather(logits, e->d_logits_gather, cnt, ncclHalf, e->comm, st));
+            }
+            V = e->vocab_local * e->cfg.tp;
+            gather_vocab_kernel<<<std::min<size_t>(1024, (cnt * e->cfg.tp / 8 + 255) / 256), 256, 0, st>>>(
+                e->d_logits_full, e->d_logits_gather, n, e->vocab_local, e->cfg.tp);
+            TM_HIP_CHECK(hipGetLastError());
+            lg = e->d_logits_full;
+        }
+        TM_PROF(P_SAMPLE, TM_TRY(launch_sample_uniform(e->d_u + slot, e->d_seed + slot, k_len, n, st)));
+        // static batch with tm_engine_set_logprobs: the kept candidates' logprobs of this step join the record of (slot, step)
+        // continuous batching with tm_engine_request_logprobs: the record of (slot, this step), handed to the host behind the step
+        const bool           lpr_cb = e->sched && e->cb_logprobs_on;
+        const bool           lpr    = (e->logprobs_on && !e->sched) || lpr_cb;
+        const SampleLogprobs lp = lpr_cb ? SampleLogprobs{e->d_cb_lp_vals, e->d_cb_lp_idx, e->d_cb_lp_num, e->d_cb_lp_sel, kMaxLogProb, nullptr, 0, 1, slot, 1}
+                                         : SampleLogprobs{e->d_lpr_vals, e->d_lpr_idx, e->d_lpr_num, e->d_lpr_sel, e->logprobs_n, e->d_step, 1, e->max_new,
+                                                          slot, e->max_new};
+        TM_PROF(P_SAMPLE, TM_TRY(launch_sample(ids, lpr ? e->d_kept + slot : nullptr, lg, n, V, V, e->d_temp + slot, e->d_topk + slot,
+                                               e->d_topp + slot, e->d_minp + slot, e->d_u + slot, e->d_sample_ws, st, lpr ? &lp : nullptr)));
+    }
+    else if (!e->use_comm) {
+        TM_PROF(P_SAMPLE, TM_TRY(launch_argmax(ids, nullptr, logits, n, e->vocab_local, e->vocab_local, 0, st)));
+    }
+    else {
+        TM_TRY(launch_argmax(ids, e->d_argmax_val, logits, n, e->vocab_local, e->vocab_local, e->cfg.rank * e->vocab_local, st));
+        pack_candidates_kernel<<<(n + 63) / 64, 64, 0, st>>>(e->d_cand, ids, e->d_argmax_val, n);
+        TM_HIP_CHECK(hipGetLastError());
+        if (e->p2p_ready) {
+            half_t*   data[8];
+            uint32_t* flags[8];
+            p2p_tables(e, data, flags);
+            TM_TRY(launch_p2p_allgather(data, flags, e->cfg.tp, e->cfg.rank, e->p2p_state, (size_t)e->p2p_rows * e->hidden, e->d_cand,
+                                        e->d_cand_all, n * 2, st));
+        }
+        else {
+            TM_NCCL_CHECK(ncclAllGather(e->d_cand, e->d_cand_all, (size_t)n * 2, ncclFloat, e->comm, st));
+        }
+        pick_kernel<<<(n + 63) / 64, 64, 0, st>>>(ids, e->d_cand_all, e->cfg.tp, n);
+        TM_HIP_CHECK(hipGetLastError());
+    }
+    return 0;
+}
+
 // One forward over M tokens.  decode: one token per sequence (cu_q = 0..B); prefill: nseq sequences.
 // Mixed forward (continuous batching, the reference's unified batch: unified_attention_layer.cc:310-311 puts the decode rows
 // first): `md` != nullptr and !decode -> rows [0, md->rows) are the decode tokens of batch slots 0 .. md->rows-1 (their KV
@@ -350,6 +436,9 @@ static int linear_fold_produce(tm_engine* e, LinearSlots& l, const half_t* x, in
 int forward(tm_engine* e, const int* d_ids, int M, int nseq, bool decode, int max_q_len, int max_k_len,
                    int kflat_stride, int slot0, const MixedDecode* md)
 {
+    if (e->lm) {  // layer-list model family (engine_layered.hip): same batch description, its own layer loop
+        return layered_forward(e, d_ids, M, nseq, decode, max_q_len, max_k_len, slot0, md);
+    }
     const tm_model_config& m = e->cfg.model;
     hipStream_t            st = e->stream;
     const int              nd = md ? md->rows : 0;  // leading decode rows of a mixed forward
@@ -536,83 +625,8 @@ int forward(tm_engine* e, const int* d_ids, int M, int nseq, bool decode, int ma
     auto head = [&](const half_t* hx, int n, int slot, const int* ids_in, const int* cu_q, int ntok, const int* k_len,
                     const int* active = nullptr) -> int {
         half_t* logits = e->d_logits + (size_t)slot * e->vocab_local;
-        int*    ids    = e->d_next_ids + slot;
         TM_PROF(P_LM_HEAD, TM_TRY(linear_plain(e, e->output, hx, e->hidden, logits, e->vocab_local, n, false)));
-        if (e->logits_on) {
-            // the tokens this forward consumed join the slots' seen masks, then penalty / bans on the (local) logits
-            uint32_t* seen = e->d_seen + (size_t)slot * e->seen_words;
-            TM_PROF(P_SAMPLE, TM_TRY(launch_seen_update(seen, e->seen_words, ids_in, cu_q, n, ntok, m.vocab, st, active)));
-            TM_PROF(P_SAMPLE, TM_TRY(launch_logits_process(logits, n, e->vocab_local, e->vocab_local,
-                                                           e->vocab_local < m.vocab ? e->cfg.rank * e->vocab_local : 0, seen,
-                                                           e->seen_words, e->d_lp_rep + slot, e->d_lp_ban + slot * kMaxBadIds,
-                                                           e->d_lp_end + slot * kMaxEndIds, k_len, e->d_lp_minlen + slot, st)));
-        }
-        if (e->sampling_on && (!e->use_comm || ((e->comm || e->p2p_ready) && e->d_logits_full))) {
-            // parameters are indexed by batch slot, the counter (context length) by the row of this forward
-            const half_t* lg = logits;
-            int           V  = e->vocab_local;
-            if (e->use_comm) {
-                // tp > 1: the vocabulary shards are all-gathered into full rows (the reference gathers the logits too,
-                // models/language_model.cc:304-333) and EVERY rank draws from the same distribution with the same Philox
-                // number -> the same token everywhere, no further exchange
-                const size_t cnt = (size_t)n * e->vocab_local;
-                if (!e->comm) {
-                    // native communicator alone: the shards travel through the P2P segments, as many whole rows per exchange as
-                    // one segment buffer holds; rank q's rows land in its [n][vocab / tp] plane of d_logits_gather
-                    half_t*   data[8];
-                    uint32_t* flags[8];
-                    p2p_tables(e, data, flags);
-                    const size_t tile = (size_t)e->p2p_rows * e->hidden;  // fp16 elements of one segment buffer
-                    const int    per  = (int)std::min<size_t>(n, tile / e->vocab_local);
-                    TM_REQUIRE(per >= 1, "native communicator: one logits row does not fit a segment buffer (export more rows)");
-                    for (int r0 = 0; r0 < n; r0 += per) {
-                        const int rows = std::min(per, n - r0);
-                        TM_TRY(launch_p2p_allgather(data, flags, e->cfg.tp, e->cfg.rank, e->p2p_state, tile, logits + (size_t)r0 * e->vocab_local,
-                                                    e->d_logits_gather + (size_t)r0 * e->vocab_local, rows * e->vocab_local / 2, st,
-                                                    cnt / 2));
-                    }
-                }
-                else {
-                    TM_NCCL_CHECK(ncclAllGather(logits, e->d_logits_gather, cnt, ncclHalf, e->comm, st));
-                }
-                V = e->vocab_local * e->cfg.tp;
-                gather_vocab_kernel<<<std::min<size_t>(1024, (cnt * e->cfg.tp / 8 + 255) / 256), 256, 0, st>>>(
-                    e->d_logits_full, e->d_logits_gather, n, e->vocab_local, e->cfg.tp);
-                TM_HIP_CHECK(hipGetLastError());
-                lg = e->d_logits_full;
-            }
-            TM_PROF(P_SAMPLE, TM_TRY(launch_sample_uniform(e->d_u + slot, e->d_seed + slot, k_len, n, st)));
-            // static batch with tm_engine_set_logprobs: the kept candidates' logprobs of this step join the record of (slot, step)
-            // continuous batching with tm_engine_request_logprobs: the record of (slot, this step), handed to the host behind the step
-            const bool           lpr_cb = e->sched && e->cb_logprobs_on;
-            const bool           lpr    = (e->logprobs_on && !e->sched) || lpr_cb;
-            const SampleLogprobs lp = lpr_cb ? SampleLogprobs{e->d_cb_lp_vals, e->d_cb_lp_idx, e->d_cb_lp_num, e->d_cb_lp_sel, kMaxLogProb, nullptr, 0, 1, slot, 1}
-                                             : SampleLogprobs{e->d_lpr_vals, e->d_lpr_idx, e->d_lpr_num, e->d_lpr_sel, e->logprobs_n, e->d_step, 1, e->max_new,
-                                                              slot, e->max_new};
-            TM_PROF(P_SAMPLE, TM_TRY(launch_sample(ids, lpr ? e->d_kept + slot : nullptr, lg, n, V, V, e->d_temp + slot, e->d_topk + slot,
-                                                   e->d_topp + slot, e->d_minp + slot, e->d_u + slot, e->d_sample_ws, st, lpr ? &lp : nullptr)));
-        }
-        else if (!e->use_comm) {
-            TM_PROF(P_SAMPLE, TM_TRY(launch_argmax(ids, nullptr, logits, n, e->vocab_local, e->vocab_local, 0, st)));
-        }
-        else {
-            TM_TRY(launch_argmax(ids, e->d_argmax_val, logits, n, e->vocab_local, e->vocab_local, e->cfg.rank * e->vocab_local, st));
-            pack_candidates_kernel<<<(n + 63) / 64, 64, 0, st>>>(e->d_cand, ids, e->d_argmax_val, n);
-            TM_HIP_CHECK(hipGetLastError());
-            if (e->p2p_ready) {
-                half_t*   data[8];
-                uint32_t* flags[8];
-                p2p_tables(e, data, flags);
-                TM_TRY(launch_p2p_allgather(data, flags, e->cfg.tp, e->cfg.rank, e->p2p_state, (size_t)e->p2p_rows * e->hidden, e->d_cand,
-                                            e->d_cand_all, n * 2, st));
-            }
-            else {
-                TM_NCCL_CHECK(ncclAllGather(e->d_cand, e->d_cand_all, (size_t)n * 2, ncclFloat, e->comm, st));
-            }
-            pick_kernel<<<(n + 63) / 64, 64, 0, st>>>(ids, e->d_cand_all, e->cfg.tp, n);
-            TM_HIP_CHECK(hipGetLastError());
-        }
-        return 0;
+        return sample_rows(e, n, slot, ids_in, cu_q, ntok, k_len, active);
     };
     if (decode) {
         return head(e->d_x, nseq, slot0, d_ids, nullptr, M, e->d_k_len);

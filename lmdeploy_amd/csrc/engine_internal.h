@@ -67,6 +67,50 @@ struct Layer {
     MoeBlock                 moe;
 };
 
+// ---- layer-list model family (engine_layered.hip) ------------------------------------------------------------------------------
+// A model is a list of residual blocks, each naming its mixer, the mixer's sizes and constants, and its feed-forward; a layer may run on
+// another layer's weights with a cache of its own.  The residual stream is fp32; activations and the cache are bf16 or fp32 (dtype).
+struct LmLayer {
+    tm_layer_spec spec{};
+    int           src = 0;           // the layer whose weights this one runs on (itself unless spec.weights_of >= 0)
+    DenseWeight   qkv, up, out;      // [q | k | v] along N; up; [o | down] along K.  Owned by layer `src`
+    float *       norm1 = nullptr, *norm2 = nullptr, *sink = nullptr;
+    int           n_q = 0, n_k = 0, n_v = 0, n_att = 0;  // heads * dim, kv_heads * dim, kv_heads * vdim, heads * vdim
+    int64_t       kv_offset = 0, v_offset = 0;           // this layer's keys inside a cache block; its values behind the keys
+};
+
+struct LayeredModel {
+    tm_layered_config    cfg{};
+    std::vector<LmLayer> layers;
+    DenseWeight          head;
+    void*                embed      = nullptr;  // [vocab][width] bf16 | fp32
+    float*               final_norm = nullptr;
+    int                  elem       = 2;        // bytes of an activation / cache element
+    int                  ldw = 0, ldqkv = 0, ldcat = 0, ldv16 = 0;  // leading dimensions: normed rows, projections, [attention | ff], fp16 logits
+    int                  max_logit_rows = 0;
+    float*               d_res = nullptr;       // residual stream [max_tokens][width]
+    void *               d_h1 = nullptr, *d_h2 = nullptr, *d_qkv = nullptr, *d_cat = nullptr, *d_hn = nullptr;
+    float*               d_logits_f32 = nullptr;  // [max_logit_rows][vocab]
+    int *                d_row_seq = nullptr, *d_row_pos = nullptr, *d_iota = nullptr, *d_want = nullptr, *d_seq_slot = nullptr;
+    int *                d_step_ids = nullptr, *d_step_cu_q = nullptr, *d_step_k_len = nullptr;
+    float*               d_attn_ws = nullptr;
+    size_t               attn_ws_bytes = 0;
+    int                  decode_splits = 1;
+    int                  debug_layers  = -1;  // >= 0: the forward stops behind this many layers (parity tests read the residual stream)
+    std::map<int64_t, int> sess_len;          // open sessions (scheduler request id) -> tokens held
+};
+
+// the rows of one forward that share a block table and a (cu_q, k_len) description
+struct LmPart {
+    int             row0, rows, nseq;
+    const int*      cu_q;
+    const int*      k_len;
+    const int*      seq_slot;    // nullptr: sequence i -> table row i
+    const uint64_t* block_ptrs;
+    bool            decode;      // one row per sequence
+    int             max_q_len;
+};
+
 }  // namespace tmk
 
 using namespace tmk;
@@ -113,6 +157,7 @@ struct tm_engine {
     bool         use_comm = false;  // collectives on the data path: tp > 1 (or TM_FORCE_COMM=1: single-rank communicator,
                                     // exercises the RCCL code path on a 1-GPU box)
     std::map<std::string, Slot> slots;
+    std::unique_ptr<tmk::LayeredModel> lm;   // set: a layer-list model (tm_engine_create_layered); `layers` below stays empty
     std::vector<Layer>          layers;
     half_t*      tok_embeddings = nullptr;
     half_t*      final_norm     = nullptr;
@@ -336,6 +381,12 @@ int allreduce_rows_side(tm_engine* e, int r0, int rows, hipEvent_t* done);
 int pipe_wait(tm_engine* e, hipEvent_t done);
 int forward(tm_engine* e, const int* d_ids, int M, int nseq, bool decode, int max_q_len, int max_k_len, int kflat_stride, int slot0,
             const MixedDecode* md = nullptr);
+int sample_rows(tm_engine* e, int n, int slot, const int* ids_in, const int* cu_q, int ntok, const int* k_len, const int* active);
+int layered_forward(tm_engine* e, const int* d_ids, int M, int nseq, bool decode, int max_q_len, int max_k_len, int slot0, const MixedDecode* md);
+int layered_process_weights(tm_engine* e);
+int layered_init_synthetic(tm_engine* e, uint64_t seed);
+int layered_start(tm_engine* e);
+void layered_free(tm_engine* e);
 int device_marks_fetch(tm_engine* e, bool async);
 int device_marks_check(tm_engine* e);
 
@@ -353,6 +404,7 @@ void setup_decode(tm_engine* e, int batch);
 int prefill_slots(tm_engine* e, const int* const* seq_ids, const int* host_lens, int batch, int slot0, float* ttft_ms,
                   const MixedStep* mix = nullptr);
 bool graph_enabled(const tm_engine* e);
+int cb_enter(tm_engine* e);  // switch the engine into continuous-batching mode (scheduler, parked slots); idempotent
 int capture_step(tm_engine* e, int (*step)(tm_engine*), hipGraphExec_t* exec);
 
 }  // extern "C"

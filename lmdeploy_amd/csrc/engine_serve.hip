@@ -21,7 +21,7 @@ extern "C" {
 // k_len = 1 and its token is ignored.  A scheduler step = admit waiting requests (prefill, chunked) + one decode step
 // for everything that is running (prefill-priority, like the reference's default when new requests arrive).
 // ------------------------------------------------------------------------------------------------------------------
-static int cb_enter(tm_engine* e)
+int cb_enter(tm_engine* e)
 {
     if (e->sched) {
         return 0;
@@ -209,6 +209,10 @@ static int submit_locked(tm_engine* e, const int* host_ids, int n, int max_new_t
         return device_marks_check(e);
     }
     TM_TRY(cb_enter(e));
+    if (e->sched->n_sessions() > 0) {
+        set_last_error("caller-fed sessions are open (tm_engine_session_close first)");
+        return TM_CONFLICT;
+    }
     const int rc = e->sched->submit(host_ids, n, max_new_tokens, eos_id, req_id);
     if (rc == TM_TOO_LONG) {
         set_last_error("prompt + max_new_tokens exceeds session_len");

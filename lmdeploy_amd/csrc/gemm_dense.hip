@@ -1,0 +1,304 @@
+// Dense linears with unquantised weights: y = x . W^T for W stored [N][K] (the checkpoint's own orientation), in two number formats.
+//
+//   bf16 : weights and activations bfloat16, fp32 accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16).  Both operands are
+//          K-contiguous, so a lane's MFMA fragment (row = lane % 16, eight consecutive k at (lane / 16) * 8) is ONE 16-byte load.
+//            * skinny kernel (M <= 32, the decode step): a wave owns 16 output columns, the four waves of a workgroup split K and
+//              merge through LDS; weights stream straight from HBM into the fragments, nothing is staged.
+//            * tiled kernel (M > 32, prefill): 128 x 128 x 32 workgroup tiles staged in LDS (padded rows, no bank conflicts on the
+//              16-byte fragment reads), 2 x 2 waves of 64 x 64, next tile prefetched into registers under the MFMAs.
+//   fp32 : true 32-bit FMA arithmetic (no matrix-core shortcut, no reduced-precision mode), 64 x 64 x 16 LDS tiles, 4 x 4 per thread.
+//
+// Weights are kept as zero-padded images [Np][Kp] (Np % 128 == 0, Kp % 32 == 0): no bounds test in any inner loop.  Activation rows
+// have a leading dimension >= Kp; what lies in their pad columns only has to be finite, it meets zero weights.
+//
+// The epilogue is chosen per call (DenseEpilogue): plain store, relu(x)^2 (the squared-ReLU feed-forward), accumulate into the fp32
+// residual stream with a multiplier (resid += alpha * acc: the output projection of a residual block closes the block in the GEMM),
+// or alpha * acc as fp32 (scaled logits).
+#include "tm_kernels.h"
+
+namespace tmk {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+template<class T>
+__device__ __forceinline__ void dense_epilogue(void* y, int ldy, int m, int n, float acc, int epi, float alpha)
+{
+    const size_t i = (size_t)m * ldy + n;
+    if (epi == kDenseStore) {
+        ((T*)y)[i] = (T)acc;
+    }
+    else if (epi == kDenseRelu2) {
+        const float r = fmaxf(acc, 0.f);
+        ((T*)y)[i]    = (T)(r * r);
+    }
+    else if (epi == kDenseResidAdd) {
+        ((float*)y)[i] += alpha * acc;
+    }
+    else {
+        ((float*)y)[i] = alpha * acc;
+    }
+}
+
+// ---- bf16, M <= 32 ------------------------------------------------------------------------------------------------------------
+// grid = Np / 16 workgroups of 4 waves.  Wave w covers k-steps w, w + 4, ... (32 k each); MT = 1 or 2 row tiles of 16.
+template<int MT>
+__global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __restrict__ x, int ldx, const __bf16* __restrict__ w, int Kp,
+                                                                void* __restrict__ y, int ldy, int M, int N, int epi, float alpha)
+{
+    __shared__ float red[4][MT][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0   = blockIdx.x * 16;
+    const int r    = lane & 15, kc = (lane >> 4) * 8;
+    const __bf16* wp = w + (size_t)(n0 + r) * Kp + kc;
+    const __bf16* xp[MT];
+    bool          xin[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        xin[t] = t * 16 + r < M;
+        xp[t]  = x + (size_t)(xin[t] ? t * 16 + r : 0) * ldx + kc;
+    }
+    floatx4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 4
+    for (int k = wave * 32; k < Kp; k += 128) {
+        const bf16x8 b = *(const bf16x8*)(wp + k);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const bf16x8 a = xin[t] ? *(const bf16x8*)(xp[t] + k) : zero;
+            acc[t]         = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            red[wave][t][lane][i] = acc[t][i];
+        }
+    }
+    __syncthreads();
+    // thread (wave, lane) finishes row tile t = wave % MT ... : 256 threads cover MT * 64 * 4 values, four waves' partials each
+    for (int idx = threadIdx.x; idx < MT * 256; idx += 256) {
+        const int t = idx >> 8, l = (idx >> 2) & 63, i = idx & 3;
+        const float s = (red[0][t][l][i] + red[1][t][l][i]) + (red[2][t][l][i] + red[3][t][l][i]);
+        const int   m = t * 16 + (l >> 4) * 4 + i, n = n0 + (l & 15);  // C fragment: column = lane % 16, rows (lane / 16) * 4 + i
+        if (m < M && n < N) {
+            dense_epilogue<__bf16>(y, ldy, m, n, s, epi, alpha);
+        }
+    }
+}
+
+// ---- bf16, tiled ----------------------------------------------------------------------------------------------------------------
+constexpr int kTM = 128, kTN = 128, kTK = 32, kLdsRow = kTK + 8;  // 80-byte LDS rows: 16-byte fragment reads of 16 rows hit all banks once
+
+__global__ __launch_bounds__(256) void dense_tiled_bf16_kernel(const __bf16* __restrict__ x, int ldx, const __bf16* __restrict__ w, int Kp,
+                                                               void* __restrict__ y, int ldy, int M, int N, int epi, float alpha)
+{
+    __shared__ __attribute__((aligned(16))) __bf16 sa[2][kTM * kLdsRow];
+    __shared__ __attribute__((aligned(16))) __bf16 sb[2][kTN * kLdsRow];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m0 = blockIdx.y * kTM, n0 = blockIdx.x * kTN;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    // staging: 128 rows x 32 k = 512 16-byte vectors per operand, two per thread: vector v -> row v / 4, k chunk (v % 4) * 8
+    const int  sr0 = tid >> 2, sr1 = sr0 + 64, sk = (tid & 3) * 8;
+    const bool a0 = m0 + sr0 < M, a1 = m0 + sr1 < M;
+    const __bf16* ap0 = x + (size_t)(a0 ? m0 + sr0 : 0) * ldx + sk;
+    const __bf16* ap1 = x + (size_t)(a1 ? m0 + sr1 : 0) * ldx + sk;
+    const __bf16* bp0 = w + (size_t)(n0 + sr0) * Kp + sk;
+    const __bf16* bp1 = w + (size_t)(n0 + sr1) * Kp + sk;
+    const bf16x8  zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8        ra0, ra1, rb0, rb1;
+    auto fetch = [&](int k) {
+        ra0 = a0 ? *(const bf16x8*)(ap0 + k) : zero;
+        ra1 = a1 ? *(const bf16x8*)(ap1 + k) : zero;
+        rb0 = *(const bf16x8*)(bp0 + k);
+        rb1 = *(const bf16x8*)(bp1 + k);
+    };
+    auto stash = [&](int buf) {
+        *(bf16x8*)(&sa[buf][sr0 * kLdsRow + sk]) = ra0;
+        *(bf16x8*)(&sa[buf][sr1 * kLdsRow + sk]) = ra1;
+        *(bf16x8*)(&sb[buf][sr0 * kLdsRow + sk]) = rb0;
+        *(bf16x8*)(&sb[buf][sr1 * kLdsRow + sk]) = rb1;
+    };
+    floatx4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    const int fr = lane & 15, fk = (lane >> 4) * 8;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    const int steps = Kp / kTK;
+    for (int s = 0; s < steps; ++s) {
+        const int buf = s & 1;
+        if (s + 1 < steps) {
+            fetch((s + 1) * kTK);
+        }
+        bf16x8 fa[4], fb[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            fa[i] = *(const bf16x8*)(&sa[buf][(wm + i * 16 + fr) * kLdsRow + fk]);
+            fb[i] = *(const bf16x8*)(&sb[buf][(wn + i * 16 + fr) * kLdsRow + fk]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        if (s + 1 < steps) {
+            stash(buf ^ 1);  // the other buffer: its readers finished before the barrier that ended step s - 1
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int m = m0 + wm + i * 16 + (lane >> 4) * 4 + q, n = n0 + wn + j * 16 + (lane & 15);
+                if (m < M && n < N) {
+                    dense_epilogue<__bf16>(y, ldy, m, n, acc[i][j][q], epi, alpha);
+                }
+            }
+        }
+    }
+}
+
+// ---- fp32 -------------------------------------------------------------------------------------------------------------------------
+// 64 x 64 x 16 tiles, 256 threads, 4 x 4 outputs per thread; operands transposed into LDS ([k][row]) so that a thread's four rows /
+// columns are one 16-byte read.  fmaf in k order: the result of a row does not depend on what shares its tile.
+__global__ __launch_bounds__(256) void dense_f32_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w, int Kp,
+                                                        void* __restrict__ y, int ldy, int M, int N, int epi, float alpha)
+{
+    __shared__ __attribute__((aligned(16))) float sa[16][64 + 4];
+    __shared__ __attribute__((aligned(16))) float sb[16][64 + 4];
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    const int tr = (tid >> 4) * 4, tc = (tid & 15) * 4;
+    const int lr = tid >> 2, lk = (tid & 3) * 4;  // staging: row lr (0..63), k chunk lk (0, 4, 8, 12)
+    const bool   ain = m0 + lr < M;
+    const float* ap  = x + (size_t)(ain ? m0 + lr : 0) * ldx + lk;
+    const float* bp  = w + (size_t)(n0 + lr) * Kp + lk;
+    float        acc[4][4] = {};
+    for (int k = 0; k < Kp; k += 16) {
+        const floatx4 va = ain ? *(const floatx4*)(ap + k) : floatx4{0.f, 0.f, 0.f, 0.f};
+        const floatx4 vb = *(const floatx4*)(bp + k);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sa[lk + i][lr] = va[i];
+            sb[lk + i][lr] = vb[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            const floatx4 a = *(const floatx4*)(&sa[kk][tr]);
+            const floatx4 b = *(const floatx4*)(&sb[kk][tc]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int m = m0 + tr + i, n = n0 + tc + j;
+            if (m < M && n < N) {
+                dense_epilogue<float>(y, ldy, m, n, acc[i][j], epi, alpha);
+            }
+        }
+    }
+}
+
+// ---- weight images ----------------------------------------------------------------------------------------------------------------
+// src: bf16 [rows][cols] (checkpoint bytes) -> dst[(row0 + r) * Kp + col0 + c], T = bf16 (copy) or float (exact widening)
+template<class T>
+__global__ void dense_place_kernel(T* __restrict__ dst, int Kp, int row0, int col0, const __bf16* __restrict__ src, int rows, int cols)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < (size_t)rows * cols) {
+        const int r = (int)(i / cols), c = (int)(i % cols);
+        dst[(size_t)(row0 + r) * Kp + col0 + c] = (T)(float)src[i];
+    }
+}
+
+int dense_weight_alloc(DenseWeight& d, int K, int N, int dtype, hipStream_t st)
+{
+    TM_REQUIRE(K >= 1 && N >= 1 && (dtype == kDenseBf16 || dtype == kDenseF32), "dense weight: K, N >= 1, dtype bf16 | f32");
+    d.K     = K;
+    d.N     = N;
+    d.Kp    = (K + 31) / 32 * 32;
+    d.Np    = (N + 127) / 128 * 128;
+    d.dtype = dtype;
+    d.bytes = (size_t)d.Kp * d.Np * (dtype == kDenseF32 ? 4 : 2);
+    TM_HIP_CHECK(hipMalloc(&d.w, d.bytes));
+    TM_HIP_CHECK(hipMemsetAsync(d.w, 0, d.bytes, st));
+    return 0;
+}
+
+int dense_weight_place(DenseWeight& d, int row0, int col0, const void* src_bf16, int rows, int cols, hipStream_t st)
+{
+    TM_REQUIRE(d.w && row0 >= 0 && col0 >= 0 && row0 + rows <= d.N && col0 + cols <= d.K, "dense weight: part outside the image");
+    const size_t n = (size_t)rows * cols;
+    if (d.dtype == kDenseF32) {
+        dense_place_kernel<float><<<(n + 255) / 256, 256, 0, st>>>((float*)d.w, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols);
+    }
+    else {
+        dense_place_kernel<__bf16><<<(n + 255) / 256, 256, 0, st>>>((__bf16*)d.w, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+void dense_weight_free(DenseWeight& d)
+{
+    if (d.w) {
+        (void)hipFree(d.w);
+    }
+    d.w = nullptr;
+}
+
+int launch_dense_linear(const DenseWeight& d, const void* x, int ldx, void* y, int ldy, int M, int epi, float alpha, hipStream_t st)
+{
+    TM_REQUIRE(d.w && x && y && M >= 0 && ldx >= d.Kp && ldy >= d.N, "dense linear: operands");
+    TM_REQUIRE(epi >= kDenseStore && epi <= kDenseScaleF32, "dense linear: epilogue");
+    if (M == 0) {
+        return 0;
+    }
+    if (d.dtype == kDenseF32) {
+        TM_REQUIRE(ldx % 4 == 0, "dense linear (fp32): rows must be 16-byte aligned");
+        dense_f32_kernel<<<dim3(d.Np / 64, (M + 63) / 64), 256, 0, st>>>((const float*)x, ldx, (const float*)d.w, d.Kp, y, ldy, M, d.N, epi, alpha);
+    }
+    else {
+        TM_REQUIRE(ldx % 8 == 0, "dense linear (bf16): rows must be 16-byte aligned");
+        if (M <= 16) {
+            dense_skinny_bf16_kernel<1><<<(d.N + 15) / 16, 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy, M, d.N, epi, alpha);
+        }
+        else if (M <= 32) {
+            dense_skinny_bf16_kernel<2><<<(d.N + 15) / 16, 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy, M, d.N, epi, alpha);
+        }
+        else {
+            dense_tiled_bf16_kernel<<<dim3(d.Np / kTN, (M + kTM - 1) / kTM), 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy,
+                                                                                       M, d.N, epi, alpha);
+        }
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+}  // namespace tmk

@@ -317,4 +317,78 @@ int launch_flatten_kv(half_t*     k_out,
     return 0;
 }
 
+
+// ---- general layout: per layer and block, keys [kv_heads][block_len][dim] then values [kv_heads][block_len][vdim], bf16 | fp32 ------
+__global__ void rows_prepare_kernel(int* __restrict__ row_seq, int* __restrict__ row_pos, const int* __restrict__ cu_q,
+                                    const int* __restrict__ k_len, int nseq, int rows)
+{
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= rows) {
+        return;
+    }
+    const int base = cu_q[0];   // cu_q may count from an earlier row of the forward: row t here is row base + t there
+    int lo = 0, hi = nseq - 1;  // the sequence with cu_q[s] <= base + t < cu_q[s + 1] (empty sequences are skipped by the search)
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (cu_q[mid] - base <= t) {
+            lo = mid;
+        }
+        else {
+            hi = mid - 1;
+        }
+    }
+    row_seq[t] = lo;
+    row_pos[t] = k_len[lo] - (cu_q[lo + 1] - cu_q[lo]) + (base + t - cu_q[lo]);
+}
+
+int launch_rows_prepare(int* row_seq, int* row_pos, const int* cu_q, const int* k_len, int nseq, int rows, hipStream_t st)
+{
+    TM_REQUIRE(row_seq && row_pos && cu_q && k_len && nseq >= 1, "rows_prepare: operands");
+    if (rows > 0) {
+        rows_prepare_kernel<<<(rows + 255) / 256, 256, 0, st>>>(row_seq, row_pos, cu_q, k_len, nseq, rows);
+        TM_HIP_CHECK(hipGetLastError());
+    }
+    return 0;
+}
+
+template<class T>
+__global__ void kv_store_general_kernel(const T* __restrict__ qkv, int ld, int k_col, int v_col, GeneralAttnParams p)
+{
+    const int per = p.kv_heads * (p.dim + p.vdim);
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)p.rows * per) {
+        return;
+    }
+    const int t = (int)(i / per), c = (int)(i % per);
+    const int s = p.row_seq[t], pos = p.row_pos[t];
+    char* base = (char*)p.block_ptrs[(size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride + pos / p.block_len] + p.layer_offset;
+    const int ti = pos % p.block_len;
+    const int nk = p.kv_heads * p.dim;
+    if (c < nk) {
+        const int g = c / p.dim, d = c % p.dim;
+        ((T*)base)[((size_t)g * p.block_len + ti) * p.dim + d] = qkv[(size_t)t * ld + k_col + c];
+    }
+    else {
+        const int cv = c - nk, g = cv / p.vdim, d = cv % p.vdim;
+        ((T*)(base + p.v_offset))[((size_t)g * p.block_len + ti) * p.vdim + d] = qkv[(size_t)t * ld + v_col + cv];
+    }
+}
+
+int launch_kv_store_general(const void* qkv, int ld, int k_col, int v_col, const GeneralAttnParams& p, hipStream_t st)
+{
+    TM_REQUIRE(qkv && p.row_seq && p.row_pos && p.block_ptrs && p.block_stride >= 1, "kv_store_general: operands");
+    const size_t n = (size_t)p.rows * p.kv_heads * (p.dim + p.vdim);
+    if (n == 0) {
+        return 0;
+    }
+    if (p.elem_bytes == 2) {
+        kv_store_general_kernel<uint16_t><<<(n + 255) / 256, 256, 0, st>>>((const uint16_t*)qkv, ld, k_col, v_col, p);
+    }
+    else {
+        kv_store_general_kernel<float><<<(n + 255) / 256, 256, 0, st>>>((const float*)qkv, ld, k_col, v_col, p);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
 }  // namespace tmk

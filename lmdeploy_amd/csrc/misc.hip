@@ -290,4 +290,55 @@ int ensure_dynamic_lds(const void* kernel, int bytes)
     return 0;
 }
 
+
+template<class T>
+__global__ void embedding_f32_kernel(float* __restrict__ out, const T* __restrict__ table, const int* __restrict__ ids, int T_, int H, int vocab)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < (size_t)T_ * H) {
+        const int t = (int)(i / H), c = (int)(i % H);
+        int       id = ids[t];
+        id           = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+        out[i]       = (float)table[(size_t)id * H + c];
+    }
+}
+
+int launch_embedding_f32(float* out, const void* table, int table_elem_bytes, const int* ids, int T, int H, int vocab, hipStream_t st)
+{
+    TM_REQUIRE(out && table && ids && (table_elem_bytes == 2 || table_elem_bytes == 4), "embedding_f32: operands");
+    const size_t n = (size_t)T * H;
+    if (n == 0) {
+        return 0;
+    }
+    if (table_elem_bytes == 2) {
+        embedding_f32_kernel<__bf16><<<(n + 255) / 256, 256, 0, st>>>(out, (const __bf16*)table, ids, T, H, vocab);
+    }
+    else {
+        embedding_f32_kernel<float><<<(n + 255) / 256, 256, 0, st>>>(out, (const float*)table, ids, T, H, vocab);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+__global__ void f32_to_f16_rows_kernel(half_t* __restrict__ out, int ld, const float* __restrict__ in, int n, int V)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < (size_t)n * ld) {
+        const int r = (int)(i / ld), c = (int)(i % ld);
+        const float v = c < V ? in[(size_t)r * V + c] : -65504.f;  // pad columns can never win an arg-max
+        out[i] = (half_t)fminf(fmaxf(v, -65504.f), 65504.f);
+    }
+}
+
+int launch_f32_to_f16_rows(half_t* out, int ld, const float* in, int n, int V, hipStream_t st)
+{
+    TM_REQUIRE(out && in && ld >= V, "f32_to_f16_rows: operands");
+    const size_t cnt = (size_t)n * ld;
+    if (cnt > 0) {
+        f32_to_f16_rows_kernel<<<(cnt + 255) / 256, 256, 0, st>>>(out, ld, in, n, V);
+        TM_HIP_CHECK(hipGetLastError());
+    }
+    return 0;
+}
+
 }  // namespace tmk

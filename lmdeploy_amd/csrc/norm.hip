@@ -106,4 +106,51 @@ int launch_residual_rmsnorm(half_t*       y,
     return 0;
 }
 
+
+// ---- fp32 residual stream -----------------------------------------------------------------------------------------------------------
+// one workgroup per row: sum of squares in fp32 (per-thread partial sums in index order, then a fixed tree), two outputs from one statistic
+template<class T>
+__global__ __launch_bounds__(256) void rmsnorm_f32_kernel(T* __restrict__ y0, T* __restrict__ y1, int ldy, const float* __restrict__ x,
+                                                          const int* __restrict__ rows, const float* __restrict__ w0,
+                                                          const float* __restrict__ w1, float w_offset, float eps, int H)
+{
+    __shared__ float red[4];
+    const int    m  = blockIdx.x;
+    const float* xr = x + (size_t)(rows ? rows[m] : m) * H;
+    float        ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += 256) {
+        ss = fmaf(xr[i], xr[i], ss);
+    }
+    ss = group_sum<64>(ss);
+    if ((threadIdx.x & 63) == 0) {
+        red[threadIdx.x >> 6] = ss;
+    }
+    __syncthreads();
+    const float inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += 256) {
+        const float v = xr[i] * inv;
+        y0[(size_t)m * ldy + i] = (T)(v * (w_offset + w0[i]));
+        if (y1) {
+            y1[(size_t)m * ldy + i] = (T)(v * (w_offset + w1[i]));
+        }
+    }
+}
+
+int launch_rmsnorm_f32(void* y0, void* y1, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w0, const float* w1,
+                       float w_offset, float eps, int M, int H, hipStream_t st)
+{
+    TM_REQUIRE(y0 && x && w0 && (!y1 || w1) && ldy >= H && (out_elem_bytes == 2 || out_elem_bytes == 4), "rmsnorm_f32: operands");
+    if (M == 0) {
+        return 0;
+    }
+    if (out_elem_bytes == 2) {
+        rmsnorm_f32_kernel<__bf16><<<M, 256, 0, st>>>((__bf16*)y0, (__bf16*)y1, ldy, x, rows, w0, w1, w_offset, eps, H);
+    }
+    else {
+        rmsnorm_f32_kernel<float><<<M, 256, 0, st>>>((float*)y0, (float*)y1, ldy, x, rows, w0, w1, w_offset, eps, H);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
 }  // namespace tmk

@@ -33,6 +33,7 @@ struct SchedRequest {
     bool             running  = false;
     std::vector<int> blocks;         // KV blocks owned while running
     std::vector<int> out;            // generated tokens so far
+    bool             session  = false;  // a caller-fed sequence (open_session): no prompt, no token budget, blocks taken as it grows
     // GenerationConfig.logprobs (set_logprobs): per generated token the first lp_n kept candidates (entries beyond lp_num[t] are
     // padding), their count and the token's own logprob -- the request's logprob_vals / logprob_indexes / logprob_nums outputs
     // (src/turbomind/engine/model_request.cc:88-90)
@@ -142,6 +143,74 @@ public:
             return slot && blocks_for((int)r.prompt.size() + r.max_new) <= (int)free_blocks_.size();  // head of the line decides
         }
         return false;
+    }
+
+    // Sessions: a slot whose sequence the caller feeds step by step (scoring / replay).  Nothing is reserved at admission; grow()
+    // takes blocks from the pool when the sequence crosses a block border, close_session() returns slot and blocks.
+    // 0 ok; 2 (conflict): no free slot
+    int open_session(int64_t* id)
+    {
+        int slot = -1;
+        for (int b = 0; b < max_batch_; ++b) {
+            if (slot_req_[b] < 0) {
+                slot = b;
+                break;
+            }
+        }
+        if (slot < 0) {
+            return 2;
+        }
+        SchedRequest r;
+        r.id            = next_id_++;
+        r.session       = true;
+        r.running       = true;
+        r.slot          = slot;
+        slot_req_[slot] = r.id;
+        *id             = r.id;
+        reqs_[r.id]     = std::move(r);
+        return 0;
+    }
+    // blocks the session needs on top of what it holds to reach `tokens` tokens (-1: unknown id / beyond session_len)
+    int grow_need(int64_t id, int tokens) const
+    {
+        auto it = reqs_.find(id);
+        if (it == reqs_.end() || !it->second.session || it->second.status != 0 || tokens > session_len_) {
+            return -1;
+        }
+        const int need = blocks_for(tokens) - (int)it->second.blocks.size();
+        return need > 0 ? need : 0;
+    }
+    // false: the pool cannot hold it (nothing is taken)
+    bool grow(int64_t id, int tokens)
+    {
+        const int need = grow_need(id, tokens);
+        if (need < 0 || need > (int)free_blocks_.size()) {
+            return false;
+        }
+        SchedRequest& r = reqs_[id];
+        for (int i = 0; i < need; ++i) {
+            r.blocks.push_back(free_blocks_.back());
+            free_blocks_.pop_back();
+        }
+        return true;
+    }
+    int close_session(int64_t id)
+    {
+        auto it = reqs_.find(id);
+        if (it == reqs_.end() || !it->second.session || it->second.status != 0) {
+            return 1;
+        }
+        finish(it->second, 7);
+        reqs_.erase(it);
+        return 0;
+    }
+    int n_sessions() const
+    {
+        int n = 0;
+        for (auto& kv : reqs_) {
+            n += kv.second.session && kv.second.status == 0;
+        }
+        return n;
     }
 
     // a token was produced for the sequence in `slot`; returns true if the sequence finished (slot + blocks released)

@@ -338,6 +338,67 @@ inline uint64_t* gemm_trace_for(size_t workgroups, const char* tag = "", int gx 
     return workgroups <= kTraceMaxWorkgroups ? g_gemm_dbg : nullptr;
 }
 
+// ---- gemm_dense.hip: unquantised linears, W stored [N][K]; bf16 on the matrix cores or true fp32 ------------------------------
+enum { kDenseBf16 = 0, kDenseF32 = 1 };
+// epilogues: y = acc (activation type) | y = relu(acc)^2 | y_f32 += alpha * acc (residual stream) | y_f32 = alpha * acc
+enum { kDenseStore = 0, kDenseRelu2 = 1, kDenseResidAdd = 2, kDenseScaleF32 = 3 };
+struct DenseWeight {
+    int    K = 0, N = 0, Kp = 0, Np = 0;  // Kp = K rounded up to 32, Np = N rounded up to 128: zero-padded image [Np][Kp]
+    int    dtype = kDenseBf16;
+    void*  w     = nullptr;
+    size_t bytes = 0;
+};
+int  dense_weight_alloc(DenseWeight& d, int K, int N, int dtype, hipStream_t st);
+// rows x cols bf16 block (checkpoint orientation [out][in]) -> image rows [row0, row0 + rows), columns [col0, col0 + cols):
+// concatenation along N fuses projections of one input, along K projections that are summed
+int  dense_weight_place(DenseWeight& d, int row0, int col0, const void* src_bf16, int rows, int cols, hipStream_t st);
+void dense_weight_free(DenseWeight& d);
+// x [M][ldx] (ldx >= Kp, pad columns finite), y [M][ldy]; x / y element type = the weight's dtype unless the epilogue says fp32
+int  launch_dense_linear(const DenseWeight& d, const void* x, int ldx, void* y, int ldy, int M, int epi, float alpha, hipStream_t st);
+
+// ---- attention_general.hip: paged causal attention, any head sizes, score modifiers as parameters ------------------------------
+struct GeneralAttnParams {
+    const void*     q = nullptr;    // [rows][ldq], head h at h * dim (bf16 | fp32 by elem_bytes)
+    void*           out = nullptr;  // [rows][ldo], head h at h * vdim
+    int             ldq = 0, ldo = 0, rows = 0;
+    const int*      row_seq = nullptr;   // [rows] sequence of a row
+    const int*      row_pos = nullptr;   // [rows] its position = index of its own cache entry
+    const int*      seq_slot = nullptr;  // [nseq] block-table row of a sequence (nullptr: sequence i -> row i)
+    const uint64_t* block_ptrs = nullptr;
+    int             block_stride = 0;    // table entries per block-table row
+    int64_t         layer_offset = 0;    // bytes from a block's base to this layer's keys [kv_heads][block_len][dim]
+    int64_t         v_offset = 0;        // bytes from the keys to the values [kv_heads][block_len][vdim]
+    int             block_len = 64, elem_bytes = 2;
+    int             q_heads = 0, kv_heads = 0, dim = 0, vdim = 0;
+    float           scale = 1.f, softcap = 0.f, qtemp_coef = 0.f, qtemp_every = 1.f;
+    const float*    sink = nullptr;      // [q_heads] or nullptr
+    int             splits = 1;
+    float*          partial_o = nullptr;   // [rows][q_heads][splits][vdim]
+    float*          partial_ml = nullptr;  // [rows][q_heads][splits][2]
+    // tile kernel only: the sequences of the launch
+    int             nseq = 0, max_q_len = 0;
+    const int*      cu_q = nullptr;   // [nseq + 1] first row of every sequence
+    const int*      k_len = nullptr;  // [nseq] context length including the rows of this launch
+};
+size_t general_attention_workspace_bytes(int rows, int q_heads, int vdim, int splits);
+int    launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st);
+// dispatch: prefill portions in bf16 -> the tile kernel on the matrix cores where it serves the sizes, everything else -> the row kernel
+int    launch_general_attention(const GeneralAttnParams& p, bool prefill, hipStream_t st);
+
+// ---- norm.hip / kv_cache.hip / misc.hip: the fp32 residual stream ------------------------------------------------------------------
+// y_i[m] = x[rows ? rows[m] : m] / sqrt(mean(x^2) + eps) * (w_offset + w_i), i = 0, 1 (y1 / w1 may be nullptr): the two norms of a
+// parallel block share one statistic.  x fp32 [.][H]; y bf16 | fp32 [M][ldy]; w fp32 [H]
+int launch_rmsnorm_f32(void* y0, void* y1, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w0, const float* w1,
+                       float w_offset, float eps, int M, int H, hipStream_t st);
+// out fp32 [T][H] = table[ids[t]] (table bf16 | fp32 [vocab][H])
+int launch_embedding_f32(float* out, const void* table, int table_elem_bytes, const int* ids, int T, int H, int vocab, hipStream_t st);
+// row_seq / row_pos of the rows [0, cu_q[nseq]) of nseq sequences: position = k_len[s] - (cu_q[s + 1] - cu_q[s]) + offset in the sequence
+int launch_rows_prepare(int* row_seq, int* row_pos, const int* cu_q, const int* k_len, int nseq, int rows, hipStream_t st);
+// keys / values of the new rows -> paged cache.  qkv [rows][ld]: keys at column k_col ([kv_heads][dim]), values at v_col ([kv_heads][vdim])
+int launch_kv_store_general(const void* qkv, int ld, int k_col, int v_col, const GeneralAttnParams& layout, hipStream_t st);
+// fp32 [n][V] -> fp16 [n][ld] (the sampler's logits rows)
+int launch_f32_to_f16_rows(half_t* out, int ld, const float* in, int n, int V, hipStream_t st);
+
 // ---- misc.hip ---------------------------------------------------------------------------
 int launch_embedding(half_t* out, const half_t* table, const int* ids, int T, int H, int vocab, hipStream_t st);
 int launch_fill_uniform_f16(half_t* out, size_t n, float amp, uint32_t seed, hipStream_t st);  // tuner stand-in activations

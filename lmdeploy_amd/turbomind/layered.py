@@ -1,0 +1,232 @@
+"""Layer-list model family: decoders described layer by layer in their config.json.
+
+    {"architecture": NAME, "width", "vocab", "norm": {"eps"}, "residual_mult", "logit_scale",
+     "layers": [{"type": MIXER, "mixer": {...sizes and constants...}, "mlp": {"kind", "ff"} | null, "weights_of": j}, ...]}
+
+`FAMILIES` maps an architecture name to the reader that turns such a config into a `LayeredConfig` (the native engine's
+tm_layered_config).  Weights are one `model.safetensors` of bf16 tensors, stored [out, in] under the names the engine's slots carry
+("embed", "l<i>.norm1", "l<i>.mix.q", ..., "final.norm", "head"); they are handed over as the file's own bytes -- the engine builds
+its images (fused projections, fp32 copies for dtype float32) on the device.  No torch in this module: a command-line tool that
+only replays tokens starts in a fraction of a second.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import json
+import mmap
+import os
+import struct
+from dataclasses import dataclass, field
+from typing import Sequence
+
+import numpy as np
+
+from .. import _ffi
+from .engine import Engine
+
+MIXER_ATTENTION = 1
+MLP_NONE, MLP_DENSE = 0, 1
+ACT_RELU2 = 0
+DTYPES = {'bfloat16': 0, 'bf16': 0, 'float32': 1, 'f32': 1}
+
+
+@dataclass
+class LayerSpec:
+    mixer: int = MIXER_ATTENTION
+    weights_of: int = -1
+    heads: int = 1
+    kv_heads: int = 1
+    dim: int = 64
+    vdim: int = 64
+    scale: float = 1.0
+    softcap: float = 0.0          # <= 0: scores are not capped
+    qtemp_coef: float = 0.0       # 0: no query temperature
+    qtemp_every: float = 1.0
+    sink: bool = False
+    mlp: int = MLP_NONE
+    ff: int = 0
+    act: int = ACT_RELU2
+
+
+@dataclass
+class LayeredConfig:
+    arch: str
+    width: int
+    vocab: int
+    layers: list = field(default_factory=list)
+    norm_eps: float = 1e-5
+    norm_offset: float = 0.0      # weights stored around zero: 1.0
+    residual_mult: float = 1.0
+    logit_scale: float = 1.0
+    eos_token_id: int | None = None
+    max_position_embeddings: int = 8192
+
+    def native(self, dtype: str):
+        """(tm_layered_config, keep-alive array)"""
+        arr = (_ffi.LayerSpec * len(self.layers))(*[
+            _ffi.LayerSpec(s.mixer, s.weights_of, s.heads, s.kv_heads, s.dim, s.vdim, s.scale, s.softcap, s.qtemp_coef, s.qtemp_every,
+                           int(s.sink), s.mlp, s.ff, s.act) for s in self.layers])
+        return _ffi.LayeredConfig(self.width, self.vocab, len(self.layers), arr, self.norm_eps, self.norm_offset, self.residual_mult,
+                                  self.logit_scale, DTYPES[dtype]), arr
+
+    def tensor_shapes(self) -> dict:
+        """{tensor name: shape} a checkpoint of this config holds"""
+        W, out = self.width, {'embed': (self.vocab, self.width), 'final.norm': (self.width,), 'head': (self.vocab, self.width)}
+        for i, s in enumerate(self.layers):
+            if s.weights_of >= 0:
+                continue
+            p = f'l{i}.'
+            out[p + 'norm1'] = (W,)
+            out[p + 'mix.q'], out[p + 'mix.k'] = (s.heads * s.dim, W), (s.kv_heads * s.dim, W)
+            out[p + 'mix.v'], out[p + 'mix.o'] = (s.kv_heads * s.vdim, W), (W, s.heads * s.vdim)
+            if s.sink:
+                out[p + 'mix.sink'] = (s.heads,)
+            if s.mlp:
+                out[p + 'norm2'], out[p + 'mlp.up'], out[p + 'mlp.down'] = (W,), (s.ff, W), (W, s.ff)
+        return out
+
+
+def _fokonex(c: dict) -> LayeredConfig:
+    """Fokonex: parallel residual blocks with two norms of the same input (weights stored around zero), attention without rotation --
+    positions enter through a logarithmic query temperature -- with capped scores and a per-head sink logit, squared-ReLU
+    feed-forward, scaled logits.  Layers may run on an earlier layer's weights."""
+    layers = []
+    for i, L in enumerate(c['layers']):
+        if L['type'] != 'attention':
+            raise NotImplementedError(f'layer {i}: mixer {L["type"]!r}')
+        m, mlp = L['mixer'], L.get('mlp')
+        if mlp is not None and mlp.get('kind') != 'dense':
+            raise NotImplementedError(f'layer {i}: feed-forward kind {mlp.get("kind")!r}')
+        qt = m.get('q_temp') or {}
+        layers.append(LayerSpec(mixer=MIXER_ATTENTION, weights_of=int(L.get('weights_of', -1)), heads=int(m['heads']),
+                                kv_heads=int(m['kv_heads']), dim=int(m['dim']), vdim=int(m['vdim']), scale=float(m['scale']),
+                                softcap=float(m.get('softcap') or 0.0), qtemp_coef=float(qt.get('coef') or 0.0),
+                                qtemp_every=float(qt.get('every') or 1.0), sink=True, mlp=MLP_DENSE if mlp is not None else MLP_NONE,
+                                ff=int(mlp['ff']) if mlp is not None else 0, act=ACT_RELU2))
+    return LayeredConfig(arch='Fokonex', width=int(c['width']), vocab=int(c['vocab']), layers=layers,
+                         norm_eps=float(c['norm']['eps']), norm_offset=1.0, residual_mult=float(c['residual_mult']),
+                         logit_scale=float(c['logit_scale']), eos_token_id=c.get('eos_token_id'))
+
+
+FAMILIES = {'Fokonex': _fokonex}
+
+
+def is_layered(model_path: str) -> bool:
+    try:
+        with open(os.path.join(model_path, 'config.json')) as f:
+            return json.load(f).get('architecture') in FAMILIES
+    except (OSError, ValueError):
+        return False
+
+
+def read_layered_config(model_path: str) -> LayeredConfig:
+    with open(os.path.join(model_path, 'config.json')) as f:
+        c = json.load(f)
+    arch = c.get('architecture')
+    if arch not in FAMILIES:
+        raise NotImplementedError(f'architecture {arch!r}: known layer-list families are {sorted(FAMILIES)}')
+    return FAMILIES[arch](c)
+
+
+def read_safetensors(path: str) -> dict:
+    """{name: (dtype string, shape, bytes view)} of one safetensors file: 8-byte little-endian header length, JSON header
+    (name -> dtype, shape, data_offsets), then the data.  The views point into a read-only mapping of the file."""
+    f = open(path, 'rb')
+    mm = mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_READ)
+    n, = struct.unpack('<Q', mm[:8])
+    header = json.loads(mm[8:8 + n].decode('utf-8'))
+    view = memoryview(mm)
+    out = {}
+    for name, t in header.items():
+        if name == '__metadata__':
+            continue
+        lo, hi = t['data_offsets']
+        out[name] = (t['dtype'], tuple(t['shape']), view[8 + n + lo:8 + n + hi])
+    return out
+
+
+class LayeredEngine(Engine):
+    """The native engine running a layer-list model.  Static batch, continuous batching, sampling and the engine thread are the
+    base class's; this adds the checkpoint hand-off and the sessions (caller-fed tokens -> logits)."""
+
+    def __init__(self, model: LayeredConfig, *, dtype: str = 'bfloat16', device: int = 0, max_batch_size: int = 64,
+                 session_len: int = 2048, cache_max_entry_count: float = 0.8, cache_blocks: int = 0,
+                 max_prefill_token_num: int = 8192, use_graph: int = 1):
+        self._lib = _ffi.load()
+        self.model = model
+        self.dtype = dtype
+        self.cfg = _ffi.EngineConfig(_ffi.ModelConfig(), 1, 0, device, max_batch_size, session_len, 0, 64, cache_max_entry_count,
+                                     cache_blocks, max_prefill_token_num, 0, use_graph)
+        self.cfg.model.vocab, self.cfg.model.hidden, self.cfg.model.layers = model.vocab, model.width, len(model.layers)
+        native, self._keep = model.native(dtype)
+        self._h = C.c_void_p()
+        _ffi.check(self._lib.tm_engine_create_layered(C.byref(self._h), C.byref(self.cfg), C.byref(native)))
+        self.batch = 0
+        self.max_new = 0
+
+    def load_checkpoint(self, model_path: str):
+        tensors = read_safetensors(os.path.join(model_path, 'model.safetensors'))
+        for name, shape in self.model.tensor_shapes().items():
+            if name not in tensors:
+                raise KeyError(f'{model_path}: tensor {name} is missing')
+            dt, shp, data = tensors[name]
+            if dt != 'BF16' or tuple(shp) != tuple(shape):
+                raise ValueError(f'{name}: {dt} {shp} in the file, the config says BF16 {shape}')
+            buf = np.frombuffer(data, np.uint8)
+            _ffi.check(self._lib.tm_engine_weight_copy(self._h, name.encode(), buf.ctypes.data, buf.nbytes))
+        _ffi.check(self._lib.tm_engine_process_weights(self._h))
+
+    def load_weights(self, slots: dict):
+        """slots: {tensor name: uint16 array holding bf16 bits}"""
+        for name, arr in slots.items():
+            arr = np.ascontiguousarray(arr)
+            _ffi.check(self._lib.tm_engine_weight_copy(self._h, name.encode(), arr.ctypes.data, arr.nbytes))
+        _ffi.check(self._lib.tm_engine_process_weights(self._h))
+
+    # ---- sessions ---------------------------------------------------------------------------------
+    def open_session(self) -> int:
+        sid = C.c_int64(0)
+        _ffi.check(self._lib.tm_engine_session_open(self._h, C.byref(sid)))
+        return sid.value
+
+    def close_session(self, session: int):
+        _ffi.check(self._lib.tm_engine_session_close(self._h, session))
+
+    def step_tokens(self, entries: Sequence) -> np.ndarray:
+        """entries: (session, tokens, want) triples -- ONE forward over the next tokens of these sessions; returns the fp32 logits of
+        the wanted places (indices into an entry's tokens), in entry order: [sum(len(want)), vocab]."""
+        keep, arr = [], (_ffi.StepEntry * len(entries))()
+        n_want = 0
+        for i, (sid, toks, want) in enumerate(entries):
+            t = np.ascontiguousarray(np.asarray(toks, np.int32))
+            w = np.ascontiguousarray(np.asarray(want if want is not None else [], np.int32))
+            keep += [t, w]
+            arr[i] = _ffi.StepEntry(int(sid), t.ctypes.data, int(t.size), w.ctypes.data if w.size else None, int(w.size))
+            n_want += int(w.size)
+        out = np.zeros((n_want, self.model.vocab), np.float32)
+        _ffi.check(self._lib.tm_engine_step_tokens(self._h, arr, len(entries), out.ctypes.data if n_want else None))
+        return out
+
+    def stop_after(self, layers: int):
+        """parity tests: the next forwards stop behind `layers` layers (< 0: all)"""
+        _ffi.check(self._lib.tm_engine_debug_stop_after(self._h, int(layers)))
+
+    def fetch_residual(self, rows: int) -> np.ndarray:
+        """the fp32 residual stream of the last forward, [rows][width]"""
+        out = np.zeros((rows, self.model.width), np.float32)
+        _ffi.check(self._lib.tm_engine_debug_read(self._h, 0, rows, 0, out.ctypes.data, out.nbytes))
+        return out
+
+    def fetch_logits(self) -> np.ndarray:
+        ld = (self.model.vocab + 7) // 8 * 8
+        out = np.zeros((self.batch, ld), np.float16)
+        _ffi.check(self._lib.tm_engine_fetch_logits(self._h, out.ctypes.data))
+        return out[:, :self.model.vocab]
+
+
+def build_engine(model_path: str, *, dtype: str = 'bfloat16', **kw) -> LayeredEngine:
+    """config.json + model.safetensors of a layer-list model -> a started engine"""
+    eng = LayeredEngine(read_layered_config(model_path), dtype=dtype, **kw)
+    eng.load_checkpoint(model_path)
+    eng.start()
+    return eng
