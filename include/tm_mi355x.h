@@ -546,6 +546,53 @@ int tm_engine_step_tokens(tm_engine* e, const tm_step_entry* entries, int n_entr
  * forward is tm_engine_debug_read(what = 0) with bytes = rows * width * 4 */
 int tm_engine_debug_stop_after(tm_engine* e, int layers);
 
+/* ---- operator level of the layer-list family (what tests/test_gpu_layered.py drives) -----------------------------------------------
+ * tm_rmsnorm_f32: y_i = x / sqrt(mean(x^2) + eps) * (w_offset + w_i) for one or two weight vectors (y1 / w1 may be NULL) from ONE
+ *   statistic; x fp32 [M][H] (rows != NULL: row m is x[rows[m]]), w fp32 [H], y bf16 (out_elem_bytes 2) or fp32 (4) [M][ldy].
+ * tm_dense_*: unquantised linear, weight given in checkpoint orientation [N][K] as bf16 bits; dtype TM_DTYPE_BF16 runs on the bf16
+ *   matrix cores with fp32 accumulation, TM_DTYPE_F32 widens the weight and computes in fp32.  epilogue: 0 y = acc, 1 y = relu(acc)^2
+ *   (x's type), 2 y_f32 += alpha * acc, 3 y_f32 = alpha * acc.  ldx >= K rounded up to 32 (pad columns finite).
+ * tm_general_attention: causal attention of `rows` query rows over a paged cache with arbitrary key / value sizes; the layout of a block
+ *   is [kv_heads][64][dim] keys at layer_offset, [kv_heads][64][vdim] values at layer_offset + v_offset, elements bf16 or fp32.  With
+ *   store_kv != 0 the keys / values of the rows (kv, [rows][ldkv]: keys at column k_col, values at v_col) are written to the cache first.
+ *   Row t is token row_pos[t] of sequence row_seq[t]; block_ptrs is a rectangular table [sequence][block_stride].
+ *   score = cap(q . k * scale * (1 + qtemp_coef * ln(floor((pos + 1) / qtemp_every) + 1))); sink (fp32 [q_heads]) may be NULL.
+ *   kernel: 0 dispatch (prefill != 0: the tile kernel where it serves the sizes), 1 row kernel, 2 tile kernel (needs cu_q / k_len / nseq:
+ *   rows grouped by sequence, cu_q[nseq + 1], k_len[nseq] context lengths including the rows).  splits > 1 needs workspace of
+ *   tm_general_attention_workspace() bytes. */
+int tm_rmsnorm_f32(void* y0, void* y1, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w0, const float* w1,
+                   float w_offset, float eps, int M, int H, tm_stream_t st);
+typedef struct tm_dense tm_dense;
+int tm_dense_create(tm_dense** out, int K, int N, int dtype, const void* weight_bf16_nk, tm_stream_t st);
+int tm_dense_forward(const tm_dense* w, const void* x, int ldx, void* y, int ldy, int M, int epilogue, float alpha, tm_stream_t st);
+int tm_dense_destroy(tm_dense* w);
+typedef struct tm_general_attn {
+    const void*     q;
+    void*           out;
+    int             ldq, ldo, rows;
+    const int *     row_seq, *row_pos;
+    const uint64_t* block_ptrs;
+    int             block_stride;
+    int64_t         layer_offset, v_offset;
+    int             elem_bytes, q_heads, kv_heads, dim, vdim;
+    float           scale, softcap, qtemp_coef, qtemp_every;
+    const float*    sink;
+    int             splits;
+    void*           workspace;
+    const void*     kv;
+    int             ldkv, k_col, v_col, store_kv;
+    int             kernel, prefill, nseq, max_q_len;
+    const int *     cu_q, *k_len;
+} tm_general_attn;
+size_t tm_general_attention_workspace(int rows, int q_heads, int vdim, int splits);
+int    tm_general_attention(const tm_general_attn* a, tm_stream_t st);
+/* scheduler sessions (host-only, like the tm_sched_* calls below): open takes a slot, grow takes blocks up to `tokens` tokens
+ * (TM_OOM: the pool cannot hold it, nothing is taken), close returns slot and blocks */
+struct tm_sched;
+int tm_sched_session_open(struct tm_sched* s, int64_t* session);
+int tm_sched_session_grow(struct tm_sched* s, int64_t session, int tokens);
+int tm_sched_session_close(struct tm_sched* s, int64_t session);
+
 /* ----------------------------------------------------------------------------------------------
  * Continuous batching.  Replaces ModelRequest.forward / cancel + the engine thread's
  * schedule-forward-update loop (bind.cpp:743-793, engine/engine.cc:434-470,770-870, model_request.cc:36-135):

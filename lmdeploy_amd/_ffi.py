@@ -85,6 +85,17 @@ class StepEntry(C.Structure):
     _fields_ = [('session', c_int64), ('tokens', c_void_p), ('n_tokens', c_int), ('want', c_void_p), ('n_want', c_int)]
 
 
+class GeneralAttn(C.Structure):
+    """struct tm_general_attn"""
+    _fields_ = [('q', c_void_p), ('out', c_void_p), ('ldq', c_int), ('ldo', c_int), ('rows', c_int), ('row_seq', c_void_p),
+                ('row_pos', c_void_p), ('block_ptrs', c_void_p), ('block_stride', c_int), ('layer_offset', c_int64),
+                ('v_offset', c_int64), ('elem_bytes', c_int), ('q_heads', c_int), ('kv_heads', c_int), ('dim', c_int), ('vdim', c_int),
+                ('scale', c_float), ('softcap', c_float), ('qtemp_coef', c_float), ('qtemp_every', c_float), ('sink', c_void_p),
+                ('splits', c_int), ('workspace', c_void_p), ('kv', c_void_p), ('ldkv', c_int), ('k_col', c_int), ('v_col', c_int),
+                ('store_kv', c_int), ('kernel', c_int), ('prefill', c_int), ('nseq', c_int), ('max_q_len', c_int), ('cu_q', c_void_p),
+                ('k_len', c_void_p)]
+
+
 # name -> (restype, argtypes); every int-returning function is a tm_status
 _SIGNATURES = {
     'tm_version': (c_int, []),
@@ -180,6 +191,16 @@ _SIGNATURES = {
     'tm_engine_session_close': (c_int, [c_void_p, c_int64]),
     'tm_engine_step_tokens': (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     'tm_engine_debug_stop_after': (c_int, [c_void_p, c_int]),
+    'tm_rmsnorm_f32': (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_int, c_int,
+                               c_void_p]),
+    'tm_dense_create': (c_int, [POINTER(c_void_p), c_int, c_int, c_int, c_void_p, c_void_p]),
+    'tm_dense_forward': (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
+    'tm_dense_destroy': (c_int, [c_void_p]),
+    'tm_general_attention_workspace': (c_size_t, [c_int, c_int, c_int, c_int]),
+    'tm_general_attention': (c_int, [POINTER(GeneralAttn), c_void_p]),
+    'tm_sched_session_open': (c_int, [c_void_p, POINTER(c_int64)]),
+    'tm_sched_session_grow': (c_int, [c_void_p, c_int64, c_int]),
+    'tm_sched_session_close': (c_int, [c_void_p, c_int64]),
     'tm_comm_unique_id': (c_int, [c_void_p]),
     'tm_engine_comm_init': (c_int, [c_void_p, c_void_p]),
     'tm_engine_weight_bytes': (c_int64, [c_void_p, c_char_p]),

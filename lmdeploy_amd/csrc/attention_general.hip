@@ -246,9 +246,216 @@ int launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st)
     return 0;
 }
 
+
+// ---- tile kernel (bf16) ---------------------------------------------------------------------------------------------------------------
+// Workgroup = 64 query rows of one sequence x one query head, four waves of 16 rows.  Per 64-key cache block a wave computes the
+// TRANSPOSED scores S^T = K Q^T (four 16-key tiles; A = key rows, B = query rows, both one 16-byte load per lane and 32 channels) so that a
+// lane ends up with 16 scores of ONE query row (row = lane % 16): the soft-max statistics are per-lane scalars (three shuffles join
+// the four lane groups), and the exponentiated accumulators ARE the B operand of O^T += V^T P^T -- the eight keys a lane group holds
+// in its two 16-key tiles are declared to be its eight k-slots, and the A operand (V^T, transposed through LDS once per workgroup and
+// block) is read in the same slot order.  No score or probability ever goes through memory.
+constexpr int kTileRows = 64, kVtStride = 72;  // V^T rows of 64 keys padded to 72 elements (144 bytes)
+
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float ga_tanh_fast(float x)
+{
+    // 1 - 2 / (exp(2x) + 1): absolute error ~1e-7, exact limits at +-inf
+    return 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f);
+}
+
+template<int DS /* 32-channel steps of the key size */, int VT /* 16-channel tiles of the value size */>
+__global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, int tiles_per_seq)
+{
+    __shared__ __attribute__((aligned(16))) __bf16 vt_s[VT * 16 * kVtStride];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+    const int s = blockIdx.x / tiles_per_seq, ti = blockIdx.x % tiles_per_seq, h = blockIdx.y;
+    const int row_base = p.cu_q[s] - p.cu_q[0];
+    const int q_len = p.cu_q[s + 1] - p.cu_q[s];
+    if (ti * kTileRows >= q_len) {
+        return;
+    }
+    const int D = p.dim, V = p.vdim;
+    const int g = h / (p.q_heads / p.kv_heads);
+    const int pos0 = p.k_len[s] - q_len;  // position of the sequence's first row in this launch
+    const int lr = lane & 15, lg = lane >> 4;
+    const int qi = ti * kTileRows + wave * 16 + lr;  // this lane's query row inside the sequence's portion
+    const bool q_ok = qi < q_len;
+    const int  pos  = pos0 + qi;
+    const uint64_t* table = p.block_ptrs + (size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    // query fragments: B operand of S^T, row = lane % 16, channels ds * 32 + (lane / 16) * 8 .. + 8
+    bf16x8 qf[DS];
+    {
+        const __bf16* q = (const __bf16*)p.q + (size_t)(row_base + (q_ok ? qi : 0)) * p.ldq + (size_t)h * D;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            const int d = ds * 32 + lg * 8;
+            qf[ds]      = (q_ok && d < D) ? *(const bf16x8*)(q + d) : zero8;
+        }
+    }
+    const float qscale = p.scale * ga_query_temp(p, pos);
+    const float cap = p.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+    float   m = -1e30f, l = 0.f;
+    floatx4 o[VT];
+#pragma unroll
+    for (int t = 0; t < VT; ++t) {
+        o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    const int last_pos = pos0 + min(q_len, (ti + 1) * kTileRows) - 1;  // the tile's last row sees keys 0 .. last_pos
+    const int nblk     = last_pos / 64 + 1;
+    for (int b = 0; b < nblk; ++b) {
+        const char*   base = (const char*)table[b] + p.layer_offset;
+        const __bf16* kb   = (const __bf16*)base + (size_t)g * 64 * D;
+        const __bf16* vb   = (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V;
+        // ---- S^T = K Q^T ----
+        floatx4 sc[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            sc[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+            const __bf16* kr = kb + (size_t)(kt * 16 + lr) * D;
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds) {
+                const int    d  = ds * 32 + lg * 8;
+                const bf16x8 kf = d < D ? *(const bf16x8*)(kr + d) : zero8;
+                sc[kt]          = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ds], sc[kt], 0, 0, 0);
+            }
+        }
+        // lane holds S[row lr][key b * 64 + kt * 16 + lg * 4 + r]
+        float bmax = -1e30f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = b * 64 + kt * 16 + lg * 4 + r;
+                float     v   = sc[kt][r] * qscale;
+                if (cap > 0.f) {
+                    v = cap * ga_tanh_fast(v * inv_cap);
+                }
+                v         = (q_ok && key <= pos) ? v : -1e30f;
+                sc[kt][r] = v;
+                bmax      = fmaxf(bmax, v);
+            }
+        }
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 16));
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32));
+        const float m_new = fmaxf(m, bmax);
+        const float alpha = __expf(m - m_new);
+        float       bsum  = 0.f;
+        bf16x8      pf[2];  // k-step ks: slots 0..3 = keys of tile 2 ks, slots 4..7 = keys of tile 2 ks + 1 (same lane group)
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float e = sc[kt][r] > -1e29f ? __expf(sc[kt][r] - m_new) : 0.f;
+                bsum += e;
+                pf[kt >> 1][(kt & 1) * 4 + r] = (__bf16)e;
+            }
+        }
+        bsum += __shfl_xor(bsum, 16);
+        bsum += __shfl_xor(bsum, 32);
+        l = l * alpha + bsum;
+        m = m_new;
+#pragma unroll
+        for (int t = 0; t < VT; ++t) {
+            o[t] *= alpha;
+        }
+        // ---- V block -> LDS, transposed: vt_s[channel][key] ----
+        __syncthreads();  // the previous block's readers are done
+        for (int idx = tid; idx < 64 * VT * 2; idx += 256) {
+            const int key = idx & 63, vc = idx >> 6;  // 8-channel chunk vc of key
+            const int v0  = vc * 8;
+            const bf16x8 x = v0 < V ? *(const bf16x8*)(vb + (size_t)key * V + v0) : zero8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                vt_s[(v0 + i) * kVtStride + key] = x[i];
+            }
+        }
+        __syncthreads();
+        // ---- O^T += V^T P^T ----
+#pragma unroll
+        for (int t = 0; t < VT; ++t) {
+            const __bf16* vr = &vt_s[(t * 16 + lr) * kVtStride];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const bf16x4 a0 = *(const bf16x4*)(vr + ks * 32 + lg * 4);
+                const bf16x4 a1 = *(const bf16x4*)(vr + ks * 32 + 16 + lg * 4);
+                const bf16x8 a  = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                o[t]            = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[ks], o[t], 0, 0, 0);
+            }
+        }
+    }
+    if (!q_ok) {
+        return;
+    }
+    float inv;
+    if (p.sink) {
+        const float sk = p.sink[h], mf = fmaxf(m, sk), a = __expf(m - mf);
+        inv            = a / (l * a + __expf(sk - mf));
+    }
+    else {
+        inv = 1.f / l;
+    }
+    // lane holds O[row lr][channel t * 16 + lg * 4 + r]
+    __bf16* out = (__bf16*)p.out + (size_t)(row_base + qi) * p.ldo + (size_t)h * V;
+#pragma unroll
+    for (int t = 0; t < VT; ++t) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int v = t * 16 + lg * 4 + r;
+            if (v < V) {
+                out[v] = (__bf16)(o[t][r] * inv);
+            }
+        }
+    }
+}
+
+bool general_attention_tiles_ok(const GeneralAttnParams& p)
+{
+    return p.elem_bytes == 2 && p.block_len == 64 && p.dim % 8 == 0 && p.vdim % 8 == 0 && p.dim <= 256 && p.vdim <= 256 && p.ldq % 8 == 0
+           && p.cu_q && p.k_len && p.nseq >= 1 && p.max_q_len >= 1 && p.splits == 1 && p.q_heads % p.kv_heads == 0;
+}
+
+template<int DS>
+static void launch_tiles_ds(const GeneralAttnParams& p, int tiles_per_seq, dim3 grid, hipStream_t st)
+{
+    switch ((p.vdim + 15) / 16) {
+#define TM_TILE_CASE(VT_) \
+    case VT_: attn_tiles_kernel<DS, VT_><<<grid, 256, 0, st>>>(p, tiles_per_seq); break;
+        TM_TILE_CASE(1) TM_TILE_CASE(2) TM_TILE_CASE(3) TM_TILE_CASE(4) TM_TILE_CASE(5) TM_TILE_CASE(6) TM_TILE_CASE(7) TM_TILE_CASE(8)
+        TM_TILE_CASE(9) TM_TILE_CASE(10) TM_TILE_CASE(11) TM_TILE_CASE(12) TM_TILE_CASE(13) TM_TILE_CASE(14) TM_TILE_CASE(15) TM_TILE_CASE(16)
+#undef TM_TILE_CASE
+    }
+}
+
+int launch_general_attention_tiles(const GeneralAttnParams& p, hipStream_t st)
+{
+    TM_REQUIRE(general_attention_tiles_ok(p), "attention tile kernel: bf16, 64-token blocks, dim and vdim multiples of 8 up to 256, sequence description");
+    if (p.rows == 0) {
+        return 0;
+    }
+    const int  tiles_per_seq = (p.max_q_len + kTileRows - 1) / kTileRows;
+    const dim3 grid(p.nseq * tiles_per_seq, p.q_heads);
+    switch ((p.dim + 31) / 32) {
+        case 1: launch_tiles_ds<1>(p, tiles_per_seq, grid, st); break;
+        case 2: launch_tiles_ds<2>(p, tiles_per_seq, grid, st); break;
+        case 3: launch_tiles_ds<3>(p, tiles_per_seq, grid, st); break;
+        case 4: launch_tiles_ds<4>(p, tiles_per_seq, grid, st); break;
+        case 5: launch_tiles_ds<5>(p, tiles_per_seq, grid, st); break;
+        case 6: launch_tiles_ds<6>(p, tiles_per_seq, grid, st); break;
+        case 7: launch_tiles_ds<7>(p, tiles_per_seq, grid, st); break;
+        default: launch_tiles_ds<8>(p, tiles_per_seq, grid, st); break;
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
 int launch_general_attention(const GeneralAttnParams& p, bool prefill, hipStream_t st)
 {
-    (void)prefill;
+    static const bool tiles_on = !getenv("TM_ATTN_TILES") || atoi(getenv("TM_ATTN_TILES")) != 0;  // A/B switch: 0 = row kernel everywhere
+    if (prefill && tiles_on && general_attention_tiles_ok(p)) {
+        return launch_general_attention_tiles(p, st);
+    }
     return launch_general_attention_rows(p, st);
 }
 

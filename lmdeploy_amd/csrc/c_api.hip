@@ -649,6 +649,106 @@ int tm_sched_create(tm_sched** out, int max_batch, int num_blocks, int session_l
     return 0;
 }
 
+// ---- operator level of the layer-list family ------------------------------------------------------------------------------------
+struct tm_dense {
+    DenseWeight w;
+};
+
+int tm_rmsnorm_f32(void* y0, void* y1, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w0, const float* w1,
+                   float w_offset, float eps, int M, int H, tm_stream_t st)
+{
+    return launch_rmsnorm_f32(y0, y1, ldy, out_elem_bytes, x, rows, w0, w1, w_offset, eps, M, H, (hipStream_t)st);
+}
+
+int tm_dense_create(tm_dense** out, int K, int N, int dtype, const void* weight_bf16_nk, tm_stream_t st)
+{
+    TM_REQUIRE(out && weight_bf16_nk, "null pointer");
+    auto* d = new tm_dense();
+    int   rc = dense_weight_alloc(d->w, K, N, dtype == TM_DTYPE_F32 ? kDenseF32 : kDenseBf16, (hipStream_t)st);
+    if (rc == 0) {
+        rc = dense_weight_place(d->w, 0, 0, weight_bf16_nk, N, K, (hipStream_t)st);
+    }
+    if (rc) {
+        dense_weight_free(d->w);
+        delete d;
+        return rc;
+    }
+    *out = d;
+    return 0;
+}
+
+int tm_dense_forward(const tm_dense* w, const void* x, int ldx, void* y, int ldy, int M, int epilogue, float alpha, tm_stream_t st)
+{
+    TM_REQUIRE(w, "null pointer");
+    return launch_dense_linear(w->w, x, ldx, y, ldy, M, epilogue, alpha, (hipStream_t)st);
+}
+
+int tm_dense_destroy(tm_dense* w)
+{
+    if (w) {
+        dense_weight_free(w->w);
+        delete w;
+    }
+    return 0;
+}
+
+size_t tm_general_attention_workspace(int rows, int q_heads, int vdim, int splits)
+{
+    return general_attention_workspace_bytes(rows, q_heads, vdim, splits);
+}
+
+int tm_general_attention(const tm_general_attn* a, tm_stream_t st)
+{
+    TM_REQUIRE(a && a->q && a->out && a->row_seq && a->row_pos && a->block_ptrs, "null pointer");
+    GeneralAttnParams p{};
+    p.q = a->q, p.out = a->out, p.ldq = a->ldq, p.ldo = a->ldo, p.rows = a->rows;
+    p.row_seq = a->row_seq, p.row_pos = a->row_pos, p.block_ptrs = a->block_ptrs, p.block_stride = a->block_stride;
+    p.layer_offset = a->layer_offset, p.v_offset = a->v_offset, p.block_len = 64, p.elem_bytes = a->elem_bytes;
+    p.q_heads = a->q_heads, p.kv_heads = a->kv_heads, p.dim = a->dim, p.vdim = a->vdim;
+    p.scale = a->scale, p.softcap = a->softcap, p.qtemp_coef = a->qtemp_coef, p.qtemp_every = a->qtemp_every, p.sink = a->sink;
+    p.nseq = a->nseq, p.max_q_len = a->max_q_len, p.cu_q = a->cu_q, p.k_len = a->k_len;
+    if (a->store_kv) {
+        TM_REQUIRE(a->kv, "store_kv without kv rows");
+        const int rc = launch_kv_store_general(a->kv, a->ldkv, a->k_col, a->v_col, p, (hipStream_t)st);
+        if (rc) {
+            return rc;
+        }
+    }
+    p.splits = a->splits > 1 ? a->splits : 1;
+    if (p.splits > 1) {
+        TM_REQUIRE(a->workspace, "splits > 1 without workspace");
+        p.partial_o  = (float*)a->workspace;
+        p.partial_ml = p.partial_o + (size_t)a->rows * a->q_heads * p.splits * a->vdim;
+    }
+    if (a->kernel == 1) {
+        return launch_general_attention_rows(p, (hipStream_t)st);
+    }
+    if (a->kernel == 2) {
+        return launch_general_attention_tiles(p, (hipStream_t)st);
+    }
+    return launch_general_attention(p, a->prefill != 0, (hipStream_t)st);
+}
+
+int tm_sched_session_open(tm_sched* s, int64_t* session)
+{
+    TM_REQUIRE(s && session, "null pointer");
+    return s->impl.open_session(session) ? TM_CONFLICT : 0;
+}
+
+int tm_sched_session_grow(tm_sched* s, int64_t session, int tokens)
+{
+    TM_REQUIRE(s, "null pointer");
+    const int need = s->impl.grow_need(session, tokens);
+    TM_REQUIRE(need >= 0, "unknown session / beyond session_len");
+    return s->impl.grow(session, tokens) ? 0 : TM_OOM;
+}
+
+int tm_sched_session_close(tm_sched* s, int64_t session)
+{
+    TM_REQUIRE(s, "null pointer");
+    return s->impl.close_session(session) ? TM_INVALID : 0;
+}
+
 int tm_sched_destroy(tm_sched* s)
 {
     delete s;

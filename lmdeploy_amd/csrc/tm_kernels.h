@@ -382,6 +382,9 @@ struct GeneralAttnParams {
 };
 size_t general_attention_workspace_bytes(int rows, int q_heads, int vdim, int splits);
 int    launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st);
+// bf16 tile kernel; TM_INVALID when the sizes are outside what it serves (general_attention_tiles_ok)
+bool   general_attention_tiles_ok(const GeneralAttnParams& p);
+int    launch_general_attention_tiles(const GeneralAttnParams& p, hipStream_t st);
 // dispatch: prefill portions in bf16 -> the tile kernel on the matrix cores where it serves the sizes, everything else -> the row kernel
 int    launch_general_attention(const GeneralAttnParams& p, bool prefill, hipStream_t st);
 

@@ -216,7 +216,7 @@ class TurbomindEngineConfig:
 
     def __post_init__(self):
         """Reference validation (lmdeploy/messages.py:345-367) ..."""
-        assert self.dtype in ['auto', 'float16', 'bfloat16']
+        assert self.dtype in ['auto', 'float16', 'bfloat16', 'float32']    # float32: layer-list models only (every operation in 32 bits)
         assert self.tp >= 1, 'tp must be a positive integer'
         assert self.ep >= 1, 'ep must be a positive integer'
         assert self.cache_max_entry_count > 0, 'invalid cache_max_entry_count'
@@ -233,8 +233,7 @@ class TurbomindEngineConfig:
         # ... plus: everything outside the hot path must be asked for explicitly and fails loudly
         if self.quant_policy == QuantPolicy.TURBO_QUANT:
             raise NotImplementedError('quant_policy=TURBO_QUANT')
-        if self.dtype == 'bfloat16':
-            raise NotImplementedError('dtype=bfloat16: the AWQ path is fp16 (lmdeploy/turbomind/converter.py:40-48)')
+        # (dtype bfloat16 / float32 belong to the layer-list model families; the pipeline refuses them for the fp16 AWQ / FP8 path)
         if self.model_format not in (None, 'awq', 'hf', 'fp8'):
             raise NotImplementedError(f'model_format={self.model_format!r}: only "awq" (W4A16 g128), "fp8" (e4m3, 128x128 '
                                       f'block scales) and "hf" (fp16)')

@@ -15,7 +15,7 @@ import numpy as np
 
 from . import _ffi
 from .messages import STATUS_TO_RESPONSE, GenerationConfig, Response, ResponseType, TurbomindEngineConfig
-from .turbomind import checkpoint
+from .turbomind import checkpoint, layered
 from .turbomind.engine import Engine
 from .turbomind.loader import export_weights
 
@@ -60,6 +60,28 @@ class Pipeline:
         self.backend_config = cfg
         self.tokenizer = None
         synthetic = model_path.startswith('synthetic:')
+        self._layered = not synthetic and layered.is_layered(model_path)
+        if self._layered:
+            # a layer-list model (config.json names one of layered.FAMILIES): bf16 (dtype 'auto' / 'bfloat16') or float32, one GPU, token-id
+            # prompts unless the folder carries a tokenizer; the same static batch / continuous batching / sampling as every other family
+            if cfg.tp != 1 or int(cfg.quant_policy) != 0 or cfg.model_format not in (None, 'hf') or cfg.dtype == 'float16':
+                raise NotImplementedError('layer-list models: tp=1, quant_policy=0, unquantised weights, dtype bfloat16 or float32')
+            self.model_cfg = layered.read_layered_config(model_path)
+            self.session_len = int(cfg.session_len or self.model_cfg.max_position_embeddings)
+            self.max_batch_size = cfg.max_batch_size or 64
+            self._group = None
+            self.engine = layered.LayeredEngine(self.model_cfg, dtype='float32' if cfg.dtype == 'float32' else 'bfloat16',
+                                                device=(cfg.devices or [0])[0], max_batch_size=self.max_batch_size,
+                                                session_len=self.session_len, cache_max_entry_count=cfg.cache_max_entry_count,
+                                                max_prefill_token_num=cfg.max_prefill_token_num or 8192)
+            self.engine.load_checkpoint(model_path)
+            if os.path.exists(os.path.join(model_path, 'tokenizer.json')) or os.path.exists(os.path.join(model_path, 'tokenizer.model')):
+                from transformers import AutoTokenizer
+                self.tokenizer = AutoTokenizer.from_pretrained(model_path)
+            self.engine.start()
+            return
+        if cfg.dtype in ('bfloat16', 'float32'):
+            raise NotImplementedError(f'dtype={cfg.dtype}: the AWQ / FP8 / fp16 path computes in fp16 (lmdeploy/turbomind/converter.py:40-48)')
         if synthetic:
             self.model_cfg = checkpoint.ModelConfig(**SYNTHETIC[model_path.split(':', 1)[1]],
                                                     quantized=cfg.model_format != 'hf',

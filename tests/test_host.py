@@ -484,7 +484,7 @@ def test_api_surface_and_validation():
     with pytest.raises(AssertionError):
         TurbomindEngineConfig(quant_policy=16)              # FP8 KV is rejected by the reference for TurboMind too
     assert TurbomindEngineConfig(model_format='fp8').model_format == 'fp8'
-    for bad in (dict(dp=2), dict(enable_prefix_caching=True), dict(dtype='bfloat16'), dict(model_format='gptq'),
+    for bad in (dict(dp=2), dict(enable_prefix_caching=True), dict(model_format='gptq'),
                 dict(cache_block_seq_len=128)):
         with pytest.raises(NotImplementedError):
             TurbomindEngineConfig(**bad)
