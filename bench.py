@@ -338,10 +338,25 @@ def main():
     ap.add_argument('--emulate-tp', type=int, default=0,
                     help='SURVEY 8(e) on a 1-GPU box: run ONE rank\'s shard of a TP=N job (heads / inter / vocab divided by N, '
                          'collectives through a 1-rank RCCL communicator): per-rank kernel time only, labelled as such')
+    ap.add_argument('--layered', action='store_true',
+                    help='instead of the headline workload: prefill and decode throughput of a layer-list model (Fokonex blocks, bf16) at the layer '
+                         'shapes of real decoders beside the fp16 Llama-family engine at equal size (lmdeploy_amd/turbomind/layered_bench.py); '
+                         'prints its own JSON line; 1 GPU')
+    ap.add_argument('--layered-sizes', default='', help='with --layered: comma-separated subset of w2048,w4096')
     ap.add_argument('--cpu-config0', action='store_true',
                     help='BASELINE.json configs[0] only: InternLM2-1.8B fp16 greedy decode on the host cores (oracle/cpu_baseline.py::run_config0, the '
                          'torch-CPU port of the reference\'s default-backend ops); prints its own JSON line; no GPU is touched')
     args = ap.parse_args()
+    if args.layered:
+        from lmdeploy_amd.turbomind import layered_bench
+        steps = 64 if args.steps == 512 else args.steps
+        batch = 32 if args.batch == 64 else args.batch
+        r = layered_bench.run(steps, args.warmup, batch, args.prompt_len, [x for x in args.layered_sizes.split(',') if x] or None)
+        emit_json({'metric': f'prefill and decode tokens/sec of a Fokonex layer-list model (bf16) beside the fp16 Llama-family engine at equal size, '
+                             f'decode batch {batch}, context {args.prompt_len}', 'value': round(next(iter(r.values()))['fokonex_bf16']['decode_tokens_per_s'], 1),
+                   'unit': 'tokens/s', 'n_gpus': 1, 'steps': steps, 'warmup': args.warmup, 'higher_is_better': True, 'dtype': 'bf16', 'data': 'synthetic',
+                   'vs_baseline': None, 'config': {'sizes': r}})
+        return
     if args.cpu_config0:
         from oracle import cpu_baseline
         b = 1 if args.batch == 64 else args.batch
