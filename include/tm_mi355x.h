@@ -553,11 +553,12 @@ int tm_engine_debug_stop_after(tm_engine* e, int layers);
  *   matrix cores with fp32 accumulation, TM_DTYPE_F32 widens the weight and computes in fp32.  epilogue: 0 y = acc, 1 y = relu(acc)^2
  *   (x's type), 2 y_f32 += alpha * acc, 3 y_f32 = alpha * acc.  ldx >= K rounded up to 32 (pad columns finite).
  * tm_general_attention: causal attention of `rows` query rows over a paged cache with arbitrary key / value sizes; the layout of a block
- *   is [kv_heads][64][dim] keys at layer_offset, [kv_heads][64][vdim] values at layer_offset + v_offset, elements bf16 or fp32.  With
+ *   is [kv_heads][64][dim] keys at layer_offset, values TRANSPOSED [kv_heads][vdim][64] at layer_offset + v_offset, elements bf16 or fp32.  With
  *   store_kv != 0 the keys / values of the rows (kv, [rows][ldkv]: keys at column k_col, values at v_col) are written to the cache first.
  *   Row t is token row_pos[t] of sequence row_seq[t]; block_ptrs is a rectangular table [sequence][block_stride].
  *   score = cap(q . k * scale * (1 + qtemp_coef * ln(floor((pos + 1) / qtemp_every) + 1))); sink (fp32 [q_heads]) may be NULL.
- *   kernel: 0 dispatch (prefill != 0: the tile kernel where it serves the sizes), 1 row kernel, 2 tile kernel (needs cu_q / k_len / nseq:
+ *   kernel: 0 dispatch (prefill != 0: the tile kernel where it serves the sizes), 1 row kernel, 3 decode kernel (bf16, one row per sequence:
+ *   row t = sequence t), 2 tile kernel (needs cu_q / k_len / nseq:
  *   rows grouped by sequence, cu_q[nseq + 1], k_len[nseq] context lengths including the rows).  splits > 1 needs workspace of
  *   tm_general_attention_workspace() bytes. */
 int tm_rmsnorm_f32(void* y0, void* y1, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w0, const float* w1,

@@ -10,9 +10,22 @@
 // position row_pos[t] and sees the cache entries 0 .. row_pos[t] of that sequence (its own key was stored before the launch).
 //   * row kernel : one wave per (row, query head, key split); lanes own keys for the scores and value channels for the output.
 //                  The decode path (few rows, long contexts: split keys + merge kernel) and the fp32 path.
-//   * tile kernel: bf16 prefill on the matrix cores -- 64 query rows of one sequence x one query head per workgroup, 64-key cache
-//                  blocks through LDS, S = Q K^T and O += P V as v_mfma_f32_16x16x32_bf16, online soft-max in fp32.
+//   * tile kernel: bf16 prefill on the matrix cores -- 64 query rows of one sequence x one query head per workgroup, four waves of 16
+//                  rows; S^T = K Q^T and O^T += V^T P^T as v_mfma_f32_16x16x32_bf16 with every operand a 16-byte load straight from the
+//                  cache (keys [token][channel], values stored transposed [channel][token]); online soft-max in fp32; no LDS, no barrier.
+//   * decode kernel: the same products with the query HEADS of one key head as the 16 rows (one row per sequence): a workgroup per
+//                  (sequence, key head, key split), its four waves take every fourth cache block and merge at the end.
+// Cache block layout per layer: keys [kv_heads][64][dim], then values [kv_heads][vdim][64].
 #include "tm_kernels.h"
+#include <stdlib.h>
+
+#define TM_TRY_RC(expr)      \
+    do {                     \
+        int _rc = (expr);    \
+        if (_rc) {           \
+            return _rc;      \
+        }                    \
+    } while (0)
 
 namespace tmk {
 
@@ -111,7 +124,7 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
     for (int b = b0; b < b1; ++b) {
         const char* base = (const char*)table[b] + p.layer_offset;
         const T*    kb   = (const T*)base + (size_t)g * p.block_len * D;
-        const T*    vb   = (const T*)(base + p.v_offset) + (size_t)g * p.block_len * V;
+        const T*    vb   = (const T*)(base + p.v_offset) + (size_t)g * p.block_len * V;  // [V][block_len]
         const int   n    = min(p.block_len, nkeys - b * p.block_len);
         for (int j0 = 0; j0 < n; j0 += 64) {
             const int  j     = j0 + lane;
@@ -132,12 +145,12 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
             const int cnt = min(64, n - j0);
             for (int jj = 0; jj < cnt; ++jj) {
                 const float w  = __shfl(pj, jj);
-                const T*    vr = vb + (size_t)(j0 + jj) * V;
+                const T*    vr = vb + (j0 + jj);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const int v = lane + 64 * c;
                     if (v < V) {
-                        o[c] = fmaf(w, (float)vr[v], o[c]);
+                        o[c] = fmaf(w, (float)vr[(size_t)v * p.block_len], o[c]);
                     }
                 }
             }
@@ -247,16 +260,14 @@ int launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st)
 }
 
 
-// ---- tile kernel (bf16) ---------------------------------------------------------------------------------------------------------------
-// Workgroup = 64 query rows of one sequence x one query head, four waves of 16 rows.  Per 64-key cache block a wave computes the
-// TRANSPOSED scores S^T = K Q^T (four 16-key tiles; A = key rows, B = query rows, both one 16-byte load per lane and 32 channels) so that a
-// lane ends up with 16 scores of ONE query row (row = lane % 16): the soft-max statistics are per-lane scalars (three shuffles join
-// the four lane groups), and the exponentiated accumulators ARE the B operand of O^T += V^T P^T -- the eight keys a lane group holds
-// in its two 16-key tiles are declared to be its eight k-slots, and the A operand (V^T, transposed through LDS once per workgroup and
-// block) is read in the same slot order.  No score or probability ever goes through memory.
-constexpr int kTileRows = 64, kVtStride = 72;  // V^T rows of 64 keys padded to 72 elements (144 bytes)
-
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+// ---- matrix-core kernels (bf16) -------------------------------------------------------------------------------------------------------
+// Per 64-key cache block a wave computes the TRANSPOSED scores S^T = K Q^T as four 16-key tiles (A = key rows, B = query rows; one
+// 16-byte load per lane and 32 channels), so that a lane ends up with 16 scores of ONE query row (row = lane % 16): the soft-max
+// statistics are per-lane scalars (two shuffles join the four lane groups) and the exponentiated accumulators ARE the B operand of
+// O^T += V^T P^T.  Which 16 keys form a tile is free: tile kt, A-row i is key (kt / 2) * 32 + (i / 4) * 8 + (kt % 2) * 4 + i % 4, which
+// leaves lane group lg with the EIGHT CONSECUTIVE keys ks * 32 + lg * 8 .. + 8 of k-step ks in its two tiles -- the A operand of the
+// second product is then one 16-byte load from the transposed values.  No score or probability ever goes through memory.
+constexpr int kTileRows = 64;
 
 __device__ __forceinline__ float ga_tanh_fast(float x)
 {
@@ -264,15 +275,83 @@ __device__ __forceinline__ float ga_tanh_fast(float x)
     return 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f);
 }
 
+// one 64-key block for 16 query rows: updates (m, l, o) of the lane's row.  qf: the rows' query fragments; limit: last visible key of
+// the lane's row (block-relative; < 0: none); kb / vb: the key head's keys [64][D] and transposed values [V][64] of this block.
+template<int DS, int VT>
+__device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[DS], const __bf16* __restrict__ kb, const __bf16* __restrict__ vb, int D, int V,
+                                              int limit, float qscale, float cap, float inv_cap, float& m, float& l, floatx4 (&o)[VT])
+{
+    const int    lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    floatx4      sc[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+        sc[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+        const __bf16* kr = kb + (size_t)((kt >> 1) * 32 + (lr >> 2) * 8 + (kt & 1) * 4 + (lr & 3)) * D;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            const int    d  = ds * 32 + lg * 8;
+            const bf16x8 kf = d < D ? *(const bf16x8*)(kr + d) : zero8;
+            sc[kt]          = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ds], sc[kt], 0, 0, 0);
+        }
+    }
+    // lane holds S[row lr][key (kt / 2) * 32 + lg * 8 + (kt % 2) * 4 + r]
+    float bmax = -1e30f;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int key = (kt >> 1) * 32 + lg * 8 + (kt & 1) * 4 + r;
+            float     v   = sc[kt][r] * qscale;
+            if (cap > 0.f) {
+                v = cap * ga_tanh_fast(v * inv_cap);
+            }
+            v         = key <= limit ? v : -1e30f;
+            sc[kt][r] = v;
+            bmax      = fmaxf(bmax, v);
+        }
+    }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 16));
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32));
+    const float m_new = fmaxf(m, bmax);
+    const float alpha = __expf(m - m_new);
+    float       bsum  = 0.f;
+    bf16x8      pf[2];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float e = sc[kt][r] > -1e29f ? __expf(sc[kt][r] - m_new) : 0.f;
+            bsum += e;
+            pf[kt >> 1][(kt & 1) * 4 + r] = (__bf16)e;
+        }
+    }
+    bsum += __shfl_xor(bsum, 16);
+    bsum += __shfl_xor(bsum, 32);
+    l = l * alpha + bsum;
+    m = m_new;
+#pragma unroll
+    for (int t = 0; t < VT; ++t) {
+        o[t] *= alpha;
+        const int     v  = t * 16 + lr;
+        const __bf16* vr = vb + (size_t)v * 64 + lg * 8;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const bf16x8 a = v < V ? *(const bf16x8*)(vr + ks * 32) : zero8;
+            o[t]           = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[ks], o[t], 0, 0, 0);
+        }
+    }
+}
+
+// Prefill: workgroup = 64 query rows of one sequence x one query head, four independent waves of 16 rows.
 template<int DS /* 32-channel steps of the key size */, int VT /* 16-channel tiles of the value size */>
 __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, int tiles_per_seq)
 {
-    __shared__ __attribute__((aligned(16))) __bf16 vt_s[VT * 16 * kVtStride];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int s = blockIdx.x / tiles_per_seq, ti = blockIdx.x % tiles_per_seq, h = blockIdx.y;
     const int row_base = p.cu_q[s] - p.cu_q[0];
     const int q_len = p.cu_q[s + 1] - p.cu_q[s];
-    if (ti * kTileRows >= q_len) {
+    if (ti * kTileRows + wave * 16 >= q_len) {
         return;
     }
     const int D = p.dim, V = p.vdim;
@@ -284,8 +363,7 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
     const int  pos  = pos0 + qi;
     const uint64_t* table = p.block_ptrs + (size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    // query fragments: B operand of S^T, row = lane % 16, channels ds * 32 + (lane / 16) * 8 .. + 8
-    bf16x8 qf[DS];
+    bf16x8 qf[DS];  // B operand of S^T: row = lane % 16, channels ds * 32 + (lane / 16) * 8 .. + 8
     {
         const __bf16* q = (const __bf16*)p.q + (size_t)(row_base + (q_ok ? qi : 0)) * p.ldq + (size_t)h * D;
 #pragma unroll
@@ -302,88 +380,12 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
     for (int t = 0; t < VT; ++t) {
         o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    const int last_pos = pos0 + min(q_len, (ti + 1) * kTileRows) - 1;  // the tile's last row sees keys 0 .. last_pos
+    const int last_pos = pos0 + min(q_len, ti * kTileRows + wave * 16 + 16) - 1;  // the wave's last row sees keys 0 .. last_pos
     const int nblk     = last_pos / 64 + 1;
     for (int b = 0; b < nblk; ++b) {
-        const char*   base = (const char*)table[b] + p.layer_offset;
-        const __bf16* kb   = (const __bf16*)base + (size_t)g * 64 * D;
-        const __bf16* vb   = (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V;
-        // ---- S^T = K Q^T ----
-        floatx4 sc[4];
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-            sc[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
-            const __bf16* kr = kb + (size_t)(kt * 16 + lr) * D;
-#pragma unroll
-            for (int ds = 0; ds < DS; ++ds) {
-                const int    d  = ds * 32 + lg * 8;
-                const bf16x8 kf = d < D ? *(const bf16x8*)(kr + d) : zero8;
-                sc[kt]          = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ds], sc[kt], 0, 0, 0);
-            }
-        }
-        // lane holds S[row lr][key b * 64 + kt * 16 + lg * 4 + r]
-        float bmax = -1e30f;
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = b * 64 + kt * 16 + lg * 4 + r;
-                float     v   = sc[kt][r] * qscale;
-                if (cap > 0.f) {
-                    v = cap * ga_tanh_fast(v * inv_cap);
-                }
-                v         = (q_ok && key <= pos) ? v : -1e30f;
-                sc[kt][r] = v;
-                bmax      = fmaxf(bmax, v);
-            }
-        }
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 16));
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 32));
-        const float m_new = fmaxf(m, bmax);
-        const float alpha = __expf(m - m_new);
-        float       bsum  = 0.f;
-        bf16x8      pf[2];  // k-step ks: slots 0..3 = keys of tile 2 ks, slots 4..7 = keys of tile 2 ks + 1 (same lane group)
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float e = sc[kt][r] > -1e29f ? __expf(sc[kt][r] - m_new) : 0.f;
-                bsum += e;
-                pf[kt >> 1][(kt & 1) * 4 + r] = (__bf16)e;
-            }
-        }
-        bsum += __shfl_xor(bsum, 16);
-        bsum += __shfl_xor(bsum, 32);
-        l = l * alpha + bsum;
-        m = m_new;
-#pragma unroll
-        for (int t = 0; t < VT; ++t) {
-            o[t] *= alpha;
-        }
-        // ---- V block -> LDS, transposed: vt_s[channel][key] ----
-        __syncthreads();  // the previous block's readers are done
-        for (int idx = tid; idx < 64 * VT * 2; idx += 256) {
-            const int key = idx & 63, vc = idx >> 6;  // 8-channel chunk vc of key
-            const int v0  = vc * 8;
-            const bf16x8 x = v0 < V ? *(const bf16x8*)(vb + (size_t)key * V + v0) : zero8;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                vt_s[(v0 + i) * kVtStride + key] = x[i];
-            }
-        }
-        __syncthreads();
-        // ---- O^T += V^T P^T ----
-#pragma unroll
-        for (int t = 0; t < VT; ++t) {
-            const __bf16* vr = &vt_s[(t * 16 + lr) * kVtStride];
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                const bf16x4 a0 = *(const bf16x4*)(vr + ks * 32 + lg * 4);
-                const bf16x4 a1 = *(const bf16x4*)(vr + ks * 32 + 16 + lg * 4);
-                const bf16x8 a  = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-                o[t]            = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[ks], o[t], 0, 0, 0);
-            }
-        }
+        const char* base = (const char*)table[b] + p.layer_offset;
+        ga_block_step<DS, VT>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D, V,
+                              q_ok ? pos - b * 64 : -1, qscale, cap, inv_cap, m, l, o);
     }
     if (!q_ok) {
         return;
@@ -410,6 +412,121 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
     }
 }
 
+// Decode: grid (sequences, kv_heads * head chunks, splits).  The 16 rows are query heads g * group + chunk * 16 + (lane % 16) of row t;
+// wave w takes the blocks b0 + w, b0 + w + 4, ... of the split; waves 1..3 hand their (m, l, O) to wave 0 through LDS.
+template<int DS, int VT>
+__global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, int chunks)
+{
+    __shared__ float ml_s[4][16][2];
+    __shared__ float o_s[3][16][VT * 16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x, g = blockIdx.y / chunks, chunk = blockIdx.y % chunks, sp = blockIdx.z;
+    const int D = p.dim, V = p.vdim, group = p.q_heads / p.kv_heads;
+    const int lr = lane & 15, lg = lane >> 4;
+    const int hg = chunk * 16 + lr;           // head inside the group
+    const bool h_ok = hg < group;
+    const int  h    = g * group + (h_ok ? hg : 0);
+    const int  s = p.row_seq[t], pos = p.row_pos[t];
+    const uint64_t* table = p.block_ptrs + (size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8 qf[DS];
+    {
+        const __bf16* q = (const __bf16*)p.q + (size_t)t * p.ldq + (size_t)h * D;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            const int d = ds * 32 + lg * 8;
+            qf[ds]      = (h_ok && d < D) ? *(const bf16x8*)(q + d) : zero8;
+        }
+    }
+    const float qscale = p.scale * ga_query_temp(p, pos);
+    const float cap = p.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+    float   m = -1e30f, l = 0.f;
+    floatx4 o[VT];
+#pragma unroll
+    for (int v = 0; v < VT; ++v) {
+        o[v] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    const int nblk = pos / 64 + 1, per = (nblk + p.splits - 1) / p.splits;
+    const int b0 = sp * per, b1 = min(nblk, b0 + per);
+    for (int b = b0 + wave; b < b1; b += 4) {
+        const char* base = (const char*)table[b] + p.layer_offset;
+        ga_block_step<DS, VT>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D, V,
+                              pos - b * 64, qscale, cap, inv_cap, m, l, o);
+    }
+    // ---- merge the four waves: common maximum, rescaled sums ----
+    if (lg == 0) {
+        ml_s[wave][lr][0] = m;
+        ml_s[wave][lr][1] = l;
+    }
+    __syncthreads();
+    const float mf = fmaxf(fmaxf(ml_s[0][lr][0], ml_s[1][lr][0]), fmaxf(ml_s[2][lr][0], ml_s[3][lr][0]));
+    const float a  = __expf(m - mf);
+    if (wave > 0) {
+#pragma unroll
+        for (int v = 0; v < VT; ++v) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                o_s[wave - 1][lr][v * 16 + lg * 4 + r] = o[v][r] * a;
+            }
+        }
+    }
+    __syncthreads();
+    if (wave > 0 || !h_ok) {
+        return;
+    }
+    float lt = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        lt += ml_s[w][lr][1] * __expf(ml_s[w][lr][0] - mf);
+    }
+#pragma unroll
+    for (int v = 0; v < VT; ++v) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int c = v * 16 + lg * 4 + r;
+            o[v][r]     = o[v][r] * a + ((o_s[0][lr][c] + o_s[1][lr][c]) + o_s[2][lr][c]);
+        }
+    }
+    if (p.splits == 1) {
+        float inv;
+        if (p.sink) {
+            const float sk = p.sink[h], m2 = fmaxf(mf, sk), a2 = __expf(mf - m2);
+            inv            = a2 / (lt * a2 + __expf(sk - m2));
+        }
+        else {
+            inv = 1.f / lt;
+        }
+        __bf16* out = (__bf16*)p.out + (size_t)t * p.ldo + (size_t)h * V;
+#pragma unroll
+        for (int v = 0; v < VT; ++v) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int c = v * 16 + lg * 4 + r;
+                if (c < V) {
+                    out[c] = (__bf16)(o[v][r] * inv);
+                }
+            }
+        }
+        return;
+    }
+    float* po = p.partial_o + (((size_t)t * p.q_heads + h) * p.splits + sp) * V;
+    float* pm = p.partial_ml + (((size_t)t * p.q_heads + h) * p.splits + sp) * 2;
+#pragma unroll
+    for (int v = 0; v < VT; ++v) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int c = v * 16 + lg * 4 + r;
+            if (c < V) {
+                po[c] = o[v][r];
+            }
+        }
+    }
+    if (lg == 0) {
+        pm[0] = mf;
+        pm[1] = lt;
+    }
+}
+
 bool general_attention_tiles_ok(const GeneralAttnParams& p)
 {
     return p.elem_bytes == 2 && p.block_len == 64 && p.dim % 8 == 0 && p.vdim % 8 == 0 && p.dim <= 256 && p.vdim <= 256 && p.ldq % 8 == 0
@@ -417,15 +534,59 @@ bool general_attention_tiles_ok(const GeneralAttnParams& p)
 }
 
 template<int DS>
-static void launch_tiles_ds(const GeneralAttnParams& p, int tiles_per_seq, dim3 grid, hipStream_t st)
+static void launch_tiles_ds(const GeneralAttnParams& p, int tiles_per_seq, dim3 grid, hipStream_t st, bool decode)
 {
     switch ((p.vdim + 15) / 16) {
-#define TM_TILE_CASE(VT_) \
-    case VT_: attn_tiles_kernel<DS, VT_><<<grid, 256, 0, st>>>(p, tiles_per_seq); break;
+#define TM_TILE_CASE(VT_)                                                           \
+    case VT_:                                                                       \
+        if (decode) {                                                               \
+            attn_decode_kernel<DS, VT_><<<grid, 256, 0, st>>>(p, tiles_per_seq);    \
+        }                                                                           \
+        else {                                                                      \
+            attn_tiles_kernel<DS, VT_><<<grid, 256, 0, st>>>(p, tiles_per_seq);     \
+        }                                                                           \
+        break;
         TM_TILE_CASE(1) TM_TILE_CASE(2) TM_TILE_CASE(3) TM_TILE_CASE(4) TM_TILE_CASE(5) TM_TILE_CASE(6) TM_TILE_CASE(7) TM_TILE_CASE(8)
         TM_TILE_CASE(9) TM_TILE_CASE(10) TM_TILE_CASE(11) TM_TILE_CASE(12) TM_TILE_CASE(13) TM_TILE_CASE(14) TM_TILE_CASE(15) TM_TILE_CASE(16)
 #undef TM_TILE_CASE
     }
+}
+
+static int launch_mfma(const GeneralAttnParams& p, int tiles_per_seq, dim3 grid, hipStream_t st, bool decode)
+{
+    switch ((p.dim + 31) / 32) {
+        case 1: launch_tiles_ds<1>(p, tiles_per_seq, grid, st, decode); break;
+        case 2: launch_tiles_ds<2>(p, tiles_per_seq, grid, st, decode); break;
+        case 3: launch_tiles_ds<3>(p, tiles_per_seq, grid, st, decode); break;
+        case 4: launch_tiles_ds<4>(p, tiles_per_seq, grid, st, decode); break;
+        case 5: launch_tiles_ds<5>(p, tiles_per_seq, grid, st, decode); break;
+        case 6: launch_tiles_ds<6>(p, tiles_per_seq, grid, st, decode); break;
+        case 7: launch_tiles_ds<7>(p, tiles_per_seq, grid, st, decode); break;
+        default: launch_tiles_ds<8>(p, tiles_per_seq, grid, st, decode); break;
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+bool general_attention_decode_ok(const GeneralAttnParams& p)
+{
+    return p.elem_bytes == 2 && p.block_len == 64 && p.dim % 8 == 0 && p.vdim % 8 == 0 && p.dim <= 256 && p.vdim <= 256 && p.ldq % 8 == 0
+           && p.q_heads % p.kv_heads == 0 && p.splits >= 1 && (p.splits == 1 || (p.partial_o && p.partial_ml));
+}
+
+int launch_general_attention_decode(const GeneralAttnParams& p, hipStream_t st)
+{
+    TM_REQUIRE(general_attention_decode_ok(p), "attention decode kernel: bf16, 64-token blocks, dim and vdim multiples of 8 up to 256");
+    if (p.rows == 0) {
+        return 0;
+    }
+    const int chunks = (p.q_heads / p.kv_heads + 15) / 16;
+    TM_TRY_RC(launch_mfma(p, chunks, dim3(p.rows, p.kv_heads * chunks, p.splits), st, true));
+    if (p.splits > 1) {
+        attn_rows_merge_kernel<__bf16><<<dim3(p.rows, p.q_heads), 64, 0, st>>>(p);
+        TM_HIP_CHECK(hipGetLastError());
+    }
+    return 0;
 }
 
 int launch_general_attention_tiles(const GeneralAttnParams& p, hipStream_t st)
@@ -434,20 +595,8 @@ int launch_general_attention_tiles(const GeneralAttnParams& p, hipStream_t st)
     if (p.rows == 0) {
         return 0;
     }
-    const int  tiles_per_seq = (p.max_q_len + kTileRows - 1) / kTileRows;
-    const dim3 grid(p.nseq * tiles_per_seq, p.q_heads);
-    switch ((p.dim + 31) / 32) {
-        case 1: launch_tiles_ds<1>(p, tiles_per_seq, grid, st); break;
-        case 2: launch_tiles_ds<2>(p, tiles_per_seq, grid, st); break;
-        case 3: launch_tiles_ds<3>(p, tiles_per_seq, grid, st); break;
-        case 4: launch_tiles_ds<4>(p, tiles_per_seq, grid, st); break;
-        case 5: launch_tiles_ds<5>(p, tiles_per_seq, grid, st); break;
-        case 6: launch_tiles_ds<6>(p, tiles_per_seq, grid, st); break;
-        case 7: launch_tiles_ds<7>(p, tiles_per_seq, grid, st); break;
-        default: launch_tiles_ds<8>(p, tiles_per_seq, grid, st); break;
-    }
-    TM_HIP_CHECK(hipGetLastError());
-    return 0;
+    const int tiles_per_seq = (p.max_q_len + kTileRows - 1) / kTileRows;
+    return launch_mfma(p, tiles_per_seq, dim3(p.nseq * tiles_per_seq, p.q_heads), st, false);
 }
 
 int launch_general_attention(const GeneralAttnParams& p, bool prefill, hipStream_t st)
@@ -455,6 +604,9 @@ int launch_general_attention(const GeneralAttnParams& p, bool prefill, hipStream
     static const bool tiles_on = !getenv("TM_ATTN_TILES") || atoi(getenv("TM_ATTN_TILES")) != 0;  // A/B switch: 0 = row kernel everywhere
     if (prefill && tiles_on && general_attention_tiles_ok(p)) {
         return launch_general_attention_tiles(p, st);
+    }
+    if (!prefill && tiles_on && general_attention_decode_ok(p)) {
+        return launch_general_attention_decode(p, st);
     }
     return launch_general_attention_rows(p, st);
 }

@@ -726,6 +726,9 @@ int tm_general_attention(const tm_general_attn* a, tm_stream_t st)
     if (a->kernel == 2) {
         return launch_general_attention_tiles(p, (hipStream_t)st);
     }
+    if (a->kernel == 3) {
+        return launch_general_attention_decode(p, (hipStream_t)st);
+    }
     return launch_general_attention(p, a->prefill != 0, (hipStream_t)st);
 }
 

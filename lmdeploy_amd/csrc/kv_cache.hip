@@ -318,7 +318,8 @@ int launch_flatten_kv(half_t*     k_out,
 }
 
 
-// ---- general layout: per layer and block, keys [kv_heads][block_len][dim] then values [kv_heads][block_len][vdim], bf16 | fp32 ------
+// ---- general layout: per layer and block, keys [kv_heads][block_len][dim] then values TRANSPOSED [kv_heads][vdim][block_len], bf16 | fp32:
+// both are then K-contiguous operands of the attention kernels' matrix products (keys: channels run fastest; values: tokens run fastest) ------
 __global__ void rows_prepare_kernel(int* __restrict__ row_seq, int* __restrict__ row_pos, const int* __restrict__ cu_q,
                                     const int* __restrict__ k_len, int nseq, int rows)
 {
@@ -370,7 +371,7 @@ __global__ void kv_store_general_kernel(const T* __restrict__ qkv, int ld, int k
     }
     else {
         const int cv = c - nk, g = cv / p.vdim, d = cv % p.vdim;
-        ((T*)(base + p.v_offset))[((size_t)g * p.block_len + ti) * p.vdim + d] = qkv[(size_t)t * ld + v_col + cv];
+        ((T*)(base + p.v_offset))[((size_t)g * p.vdim + d) * p.block_len + ti] = qkv[(size_t)t * ld + v_col + cv];
     }
 }
 

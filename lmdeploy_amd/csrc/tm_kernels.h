@@ -367,7 +367,7 @@ struct GeneralAttnParams {
     const uint64_t* block_ptrs = nullptr;
     int             block_stride = 0;    // table entries per block-table row
     int64_t         layer_offset = 0;    // bytes from a block's base to this layer's keys [kv_heads][block_len][dim]
-    int64_t         v_offset = 0;        // bytes from the keys to the values [kv_heads][block_len][vdim]
+    int64_t         v_offset = 0;        // bytes from the keys to the values, stored transposed: [kv_heads][vdim][block_len]
     int             block_len = 64, elem_bytes = 2;
     int             q_heads = 0, kv_heads = 0, dim = 0, vdim = 0;
     float           scale = 1.f, softcap = 0.f, qtemp_coef = 0.f, qtemp_every = 1.f;
@@ -382,6 +382,10 @@ struct GeneralAttnParams {
 };
 size_t general_attention_workspace_bytes(int rows, int q_heads, int vdim, int splits);
 int    launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st);
+// bf16 decode kernel on the matrix cores: one row per sequence, the query heads of a key head as the rows of the products, keys split
+// over the waves of a workgroup and over `splits` workgroups
+bool   general_attention_decode_ok(const GeneralAttnParams& p);
+int    launch_general_attention_decode(const GeneralAttnParams& p, hipStream_t st);
 // bf16 tile kernel; TM_INVALID when the sizes are outside what it serves (general_attention_tiles_ok)
 bool   general_attention_tiles_ok(const GeneralAttnParams& p);
 int    launch_general_attention_tiles(const GeneralAttnParams& p, hipStream_t st);

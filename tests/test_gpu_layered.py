@@ -86,7 +86,8 @@ def test_dense_linear_every_row_count_and_epilogue(tm, cuda, dtype):
 
 
 class Cache:
-    """a paged cache in the general layout (per block: keys [G][64][D], then values [G][64][V]) with shuffled blocks"""
+    """a paged cache in the general layout (per block: keys [G][64][D], then values transposed [G][V][64]) with shuffled blocks; the
+    tests only fix a block's size and where its values start -- every entry is written by the store path under test"""
 
     def __init__(self, dtype, G, D, V, lens, rng, extra_blocks=3):
         self.dtype, self.G, self.D, self.V, self.lens = dtype, G, D, V, lens
@@ -111,7 +112,7 @@ class Cache:
         self.eb = eb
 
 
-def run_attention(tm, cache, q, k_new, v_new, row_seq, row_pos, cu_q, k_len, spec, sink, kernel, splits=1):
+def run_attention(tm, cache, q, k_new, v_new, row_seq, row_pos, cu_q, k_len, spec, sink, kernel, splits=1, prefill=1):
     """store the new rows' keys / values, then attention; q [rows, H * D], k_new [rows, G * D], v_new [rows, G * V] (float64)"""
     dtype, H, G, D, V = cache.dtype, spec['heads'], spec['kv_heads'], spec['dim'], spec['vdim']
     rows = q.shape[0]
@@ -125,7 +126,7 @@ def run_attention(tm, cache, q, k_new, v_new, row_seq, row_pos, cu_q, k_len, spe
                          dev(np.asarray(row_pos, np.int32)).data_ptr(), cache.ptrs.data_ptr(), cache.stride, 0, cache.v_offset, cache.eb,
                          H, G, D, V, spec['scale'], spec['softcap'], spec['qtemp_coef'], spec['qtemp_every'],
                          dev(np.asarray(sink, np.float32)).data_ptr() if sink is not None else None, splits, ws.data_ptr(),
-                         qkv_d.data_ptr(), ld, H * D, H * D + G * D, 1, kernel, 1, len(cu_q) - 1, int(np.diff(cu_q).max()),
+                         qkv_d.data_ptr(), ld, H * D, H * D + G * D, 1, kernel, prefill, len(cu_q) - 1, int(np.diff(cu_q).max()),
                          dev(np.asarray(cu_q, np.int32)).data_ptr(), dev(np.asarray(k_len, np.int32)).data_ptr())
     _ffi.check(tm.tm_general_attention(C.byref(a), st()))
     return read(out, dtype)[:, :H * V]
@@ -208,6 +209,34 @@ def test_attention_finds_one_far_key_and_respects_the_causal_edge(tm, cuda, dtyp
         if hot > 0:                                                                             # the row just before must not see it
             ref = oracle_attention(q[hot - 1], keys, vals, hot - 1, spec, None)
             assert np.abs(got[hot - 1] - ref).max() <= 3e-2 and np.abs(got[hot - 1].reshape(2, 16) - vals[hot, 0]).max() > 0.2
+
+
+@pytest.mark.parametrize('dtype', [0, 1])
+@pytest.mark.parametrize('heads,kv_heads,D,V', [(4, 4, 32, 16), (6, 2, 40, 24), (40, 2, 64, 48), (8, 1, 128, 128), (2, 1, 20, 12)])
+def test_attention_decode_rows_of_unequal_sequences(tm, cuda, dtype, heads, kv_heads, D, V):
+    """one new row per sequence, contexts from 1 token to several blocks (one ends exactly at a block border, one just behind it): the
+    row kernel with and without key splits, and in bf16 the matrix-core decode kernel (query heads as rows: groups of 1, 3, 8 and 20)"""
+    spec = dict(heads=heads, kv_heads=kv_heads, dim=D, vdim=V, scale=0.2, softcap=6.0, qtemp_coef=0.5, qtemp_every=60.0)
+    rng = np.random.default_rng(heads * 7 + D + dtype)
+    hist = [0, 63, 64, 200, 330, 5]
+    lens = [n + 1 for n in hist]
+    rnd = (lambda *s: lo.bf16(rng.normal(0, 1, s))) if dtype == 0 else (lambda *s: rng.normal(0, 1, s).astype(np.float32).astype(np.float64))
+    keys, vals = [rnd(n, kv_heads, D) for n in lens], [rnd(n, kv_heads, V) for n in lens]
+    sink = rng.normal(0, 1, heads).astype(np.float32)
+    cache = Cache(dtype, kv_heads, D, V, lens, rng)
+    for s, n in enumerate(hist):
+        if n:
+            run_attention(tm, cache, rnd(n, heads * D), keys[s][:n].reshape(n, -1), vals[s][:n].reshape(n, -1), [s] * n, list(range(n)),
+                          [0] * s + [0, n] + [n] * (len(lens) - s - 1), [0] * s + [n] + [0] * (len(lens) - s - 1), spec, sink, 1)
+    q = rnd(len(lens), heads * D)
+    k_new = np.stack([keys[s][-1].reshape(-1) for s in range(len(lens))])
+    v_new = np.stack([vals[s][-1].reshape(-1) for s in range(len(lens))])
+    ref = np.stack([oracle_attention(q[s], keys[s], vals[s], hist[s], spec, sink) for s in range(len(lens))])
+    tol = (2e-2 if dtype == 0 else 2e-5) * np.abs(ref).max()
+    kernels = [(1, 1), (1, 3)] + ([(3, 1), (3, 2), (3, 8), (0, 1)] if dtype == 0 and D % 8 == 0 and V % 8 == 0 else [])
+    for kernel, splits in kernels:
+        got = run_attention(tm, cache, q, k_new, v_new, list(range(len(lens))), hist, list(range(len(lens) + 1)), lens, spec, sink, kernel, splits, prefill=0)
+        assert np.abs(got - ref).max() <= tol, (kernel, splits, np.abs(got - ref).max(), tol)
 
 
 # ---- engine -------------------------------------------------------------------------------------------------------------------------
