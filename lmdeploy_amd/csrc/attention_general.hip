@@ -267,7 +267,8 @@ int launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st)
 // O^T += V^T P^T.  Which 16 keys form a tile is free: tile kt, A-row i is key (kt / 2) * 32 + (i / 4) * 8 + (kt % 2) * 4 + i % 4, which
 // leaves lane group lg with the EIGHT CONSECUTIVE keys ks * 32 + lg * 8 .. + 8 of k-step ks in its two tiles -- the A operand of the
 // second product is then one 16-byte load from the transposed values.  No score or probability ever goes through memory.
-constexpr int kTileRows = 64;
+constexpr int   kTileRows = 64;
+constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
 
 __device__ __forceinline__ float ga_tanh_fast(float x)
 {
@@ -275,138 +276,186 @@ __device__ __forceinline__ float ga_tanh_fast(float x)
     return 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f);
 }
 
-// one 64-key block for 16 query rows: updates (m, l, o) of the lane's row.  qf: the rows' query fragments; limit: last visible key of
-// the lane's row (block-relative; < 0: none); kb / vb: the key head's keys [64][D] and transposed values [V][64] of this block.
-template<int DS, int VT>
-__device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[DS], const __bf16* __restrict__ kb, const __bf16* __restrict__ vb, int D, int V,
-                                              int limit, float qscale, float cap, float inv_cap, float& m, float& l, floatx4 (&o)[VT])
+// one 64-key block for RT tiles of 16 query rows (the lane's row of tile rt is rt * 16 + lane % 16): updates (m, l, o) of those rows.
+// Every key / value fragment is loaded ONCE and serves all RT row tiles; the value fragments are requested before the soft-max
+// arithmetic so that their latency hides under it.  qf: the rows' query fragments; limit: last visible key of the lane's rows
+// (block-relative; < 0: none); kb / vb: the key head's keys [64][D] and transposed values [V][64] of this block.
+template<int DS, int VT, int RT, bool MASK>
+__device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const __bf16* __restrict__ kb, const __bf16* __restrict__ vb, int D,
+                                              int V, const int (&limit)[RT], const float (&qscale)[RT], float cap, float inv_cap,
+                                              float (&m)[RT], float (&l)[RT], floatx4 (&o)[RT][VT])
 {
     const int    lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    floatx4      sc[4];
+    floatx4      sc[RT][4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
-        sc[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            sc[rt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
         const __bf16* kr = kb + (size_t)((kt >> 1) * 32 + (lr >> 2) * 8 + (kt & 1) * 4 + (lr & 3)) * D;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
             const int    d  = ds * 32 + lg * 8;
             const bf16x8 kf = d < D ? *(const bf16x8*)(kr + d) : zero8;
-            sc[kt]          = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ds], sc[kt], 0, 0, 0);
-        }
-    }
-    // lane holds S[row lr][key (kt / 2) * 32 + lg * 8 + (kt % 2) * 4 + r]
-    float bmax = -1e30f;
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int key = (kt >> 1) * 32 + lg * 8 + (kt & 1) * 4 + r;
-            float     v   = sc[kt][r] * qscale;
-            if (cap > 0.f) {
-                v = cap * ga_tanh_fast(v * inv_cap);
+            for (int rt = 0; rt < RT; ++rt) {
+                sc[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[rt][ds], sc[rt][kt], 0, 0, 0);
             }
-            v         = key <= limit ? v : -1e30f;
-            sc[kt][r] = v;
-            bmax      = fmaxf(bmax, v);
         }
     }
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 16));
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 32));
-    const float m_new = fmaxf(m, bmax);
-    const float alpha = __expf(m - m_new);
-    float       bsum  = 0.f;
-    bf16x8      pf[2];
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float e = sc[kt][r] > -1e29f ? __expf(sc[kt][r] - m_new) : 0.f;
-            bsum += e;
-            pf[kt >> 1][(kt & 1) * 4 + r] = (__bf16)e;
-        }
-    }
-    bsum += __shfl_xor(bsum, 16);
-    bsum += __shfl_xor(bsum, 32);
-    l = l * alpha + bsum;
-    m = m_new;
+    bf16x8 vf[VT][2];
 #pragma unroll
     for (int t = 0; t < VT; ++t) {
-        o[t] *= alpha;
         const int     v  = t * 16 + lr;
         const __bf16* vr = vb + (size_t)v * 64 + lg * 8;
+        vf[t][0]         = v < V ? *(const bf16x8*)(vr) : zero8;
+        vf[t][1]         = v < V ? *(const bf16x8*)(vr + 32) : zero8;
+    }
+    // lane holds S[row lr of tile rt][key (kt / 2) * 32 + lg * 8 + (kt % 2) * 4 + r].  From here on scores live in the log2 domain
+    // (multiplied by log2 e) so that every exponential is one v_exp_f32: the capped score is
+    //   cap2 * tanh(x / cap) = cap2 - 2 cap2 / (2^(x * 2 log2e / cap) + 1),  cap2 = cap * log2e
+    // -- five VALU operations, two of them transcendental; the kernel is bound by exactly this arithmetic.
+    bf16x8 pf[RT][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const float cap2 = cap * kLog2e, k1 = cap > 0.f ? qscale[rt] * inv_cap * (2.f * kLog2e) : qscale[rt] * kLog2e;
+        float       bmax = -1e30f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = sc[rt][kt][r] * k1;
+                if (cap > 0.f) {
+                    v = fmaf(__builtin_amdgcn_rcpf(fast_exp2(v) + 1.f), -2.f * cap2, cap2);
+                }
+                if (MASK) {
+                    const int key = (kt >> 1) * 32 + lg * 8 + (kt & 1) * 4 + r;
+                    v             = key <= limit[rt] ? v : -1e30f;
+                }
+                sc[rt][kt][r] = v;
+                bmax          = fmaxf(bmax, v);
+            }
+        }
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 16));
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32));
+        const float m_new = fmaxf(m[rt], bmax);
+        const float alpha = fast_exp2(m[rt] - m_new);
+        float       bsum  = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float e = fast_exp2(sc[rt][kt][r] - m_new);  // a masked score is -1e30: 2^(-1e30 - m) = 0 (a row sees its own key: m is finite)
+                bsum += e;
+                pf[rt][kt >> 1][(kt & 1) * 4 + r] = (__bf16)e;
+            }
+        }
+        bsum += __shfl_xor(bsum, 16);
+        bsum += __shfl_xor(bsum, 32);
+        l[rt] = l[rt] * alpha + bsum;
+        m[rt] = m_new;
+#pragma unroll
+        for (int t = 0; t < VT; ++t) {
+            o[rt][t] *= alpha;
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < VT; ++t) {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            const bf16x8 a = v < V ? *(const bf16x8*)(vr + ks * 32) : zero8;
-            o[t]           = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[ks], o[t], 0, 0, 0);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t][ks], pf[rt][ks], o[rt][t], 0, 0, 0);
+            }
         }
     }
 }
 
-// Prefill: workgroup = 64 query rows of one sequence x one query head, four independent waves of 16 rows.
-template<int DS /* 32-channel steps of the key size */, int VT /* 16-channel tiles of the value size */>
+// Prefill: workgroup = 64 * RT query rows of one sequence x one query head, four independent waves of RT tiles of 16 rows.
+template<int DS /* 32-channel steps of the key size */, int VT /* 16-channel tiles of the value size */, int RT>
 __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, int tiles_per_seq)
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int s = blockIdx.x / tiles_per_seq, ti = blockIdx.x % tiles_per_seq, h = blockIdx.y;
     const int row_base = p.cu_q[s] - p.cu_q[0];
     const int q_len = p.cu_q[s + 1] - p.cu_q[s];
-    if (ti * kTileRows + wave * 16 >= q_len) {
+    const int row0  = ti * (kTileRows * RT) + wave * (16 * RT);  // the wave's first row inside the sequence's portion
+    if (row0 >= q_len) {
         return;
     }
     const int D = p.dim, V = p.vdim;
     const int g = h / (p.q_heads / p.kv_heads);
     const int pos0 = p.k_len[s] - q_len;  // position of the sequence's first row in this launch
     const int lr = lane & 15, lg = lane >> 4;
-    const int qi = ti * kTileRows + wave * 16 + lr;  // this lane's query row inside the sequence's portion
-    const bool q_ok = qi < q_len;
-    const int  pos  = pos0 + qi;
     const uint64_t* table = p.block_ptrs + (size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    bf16x8 qf[DS];  // B operand of S^T: row = lane % 16, channels ds * 32 + (lane / 16) * 8 .. + 8
-    {
-        const __bf16* q = (const __bf16*)p.q + (size_t)(row_base + (q_ok ? qi : 0)) * p.ldq + (size_t)h * D;
+    const float cap = p.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+    bf16x8  qf[RT][DS];  // B operand of S^T: row = lane % 16, channels ds * 32 + (lane / 16) * 8 .. + 8
+    float   qscale[RT], m[RT], l[RT];
+    int     pos[RT];
+    bool    q_ok[RT];
+    floatx4 o[RT][VT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int qi = row0 + rt * 16 + lr;
+        q_ok[rt]     = qi < q_len;
+        pos[rt]      = pos0 + qi;
+        const __bf16* q = (const __bf16*)p.q + (size_t)(row_base + (q_ok[rt] ? qi : 0)) * p.ldq + (size_t)h * D;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
             const int d = ds * 32 + lg * 8;
-            qf[ds]      = (q_ok && d < D) ? *(const bf16x8*)(q + d) : zero8;
+            qf[rt][ds]  = (q_ok[rt] && d < D) ? *(const bf16x8*)(q + d) : zero8;
+        }
+        qscale[rt] = p.scale * ga_query_temp(p, pos[rt]);
+        m[rt]      = -1e30f;
+        l[rt]      = 0.f;
+#pragma unroll
+        for (int t = 0; t < VT; ++t) {
+            o[rt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
         }
     }
-    const float qscale = p.scale * ga_query_temp(p, pos);
-    const float cap = p.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
-    float   m = -1e30f, l = 0.f;
-    floatx4 o[VT];
-#pragma unroll
-    for (int t = 0; t < VT; ++t) {
-        o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-    }
-    const int last_pos = pos0 + min(q_len, ti * kTileRows + wave * 16 + 16) - 1;  // the wave's last row sees keys 0 .. last_pos
+    const int last_pos = pos0 + min(q_len, row0 + 16 * RT) - 1;  // the wave's last row sees keys 0 .. last_pos
     const int nblk     = last_pos / 64 + 1;
     for (int b = 0; b < nblk; ++b) {
         const char* base = (const char*)table[b] + p.layer_offset;
-        ga_block_step<DS, VT>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D, V,
-                              q_ok ? pos - b * 64 : -1, qscale, cap, inv_cap, m, l, o);
-    }
-    if (!q_ok) {
-        return;
-    }
-    float inv;
-    if (p.sink) {
-        const float sk = p.sink[h], mf = fmaxf(m, sk), a = __expf(m - mf);
-        inv            = a / (l * a + __expf(sk - mf));
-    }
-    else {
-        inv = 1.f / l;
-    }
-    // lane holds O[row lr][channel t * 16 + lg * 4 + r]
-    __bf16* out = (__bf16*)p.out + (size_t)(row_base + qi) * p.ldo + (size_t)h * V;
+        int         limit[RT];
 #pragma unroll
-    for (int t = 0; t < VT; ++t) {
+        for (int rt = 0; rt < RT; ++rt) {
+            limit[rt] = q_ok[rt] ? pos[rt] - b * 64 : -1;
+        }
+        const __bf16 *kb = (const __bf16*)base + (size_t)g * 64 * D, *vb = (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V;
+        if (b * 64 + 63 <= pos0 + row0) {  // every row of the wave sees the whole block (rows beyond the portion are discarded anyway)
+            ga_block_step<DS, VT, RT, false>(qf, kb, vb, D, V, limit, qscale, cap, inv_cap, m, l, o);
+        }
+        else {
+            ga_block_step<DS, VT, RT, true>(qf, kb, vb, D, V, limit, qscale, cap, inv_cap, m, l, o);
+        }
+    }
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int v = t * 16 + lg * 4 + r;
-            if (v < V) {
-                out[v] = (__bf16)(o[t][r] * inv);
+    for (int rt = 0; rt < RT; ++rt) {
+        if (!q_ok[rt]) {
+            continue;
+        }
+        float inv;
+        if (p.sink) {  // m is in the log2 domain
+            const float sk = p.sink[h] * kLog2e, mf = fmaxf(m[rt], sk), a = fast_exp2(m[rt] - mf);
+            inv            = a / (l[rt] * a + fast_exp2(sk - mf));
+        }
+        else {
+            inv = 1.f / l[rt];
+        }
+        // lane holds O[row lr][channel t * 16 + lg * 4 + r]
+        __bf16* out = (__bf16*)p.out + (size_t)(row_base + row0 + rt * 16 + lr) * p.ldo + (size_t)h * V;
+#pragma unroll
+        for (int t = 0; t < VT; ++t) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int v = t * 16 + lg * 4 + r;
+                if (v < V) {
+                    out[v] = (__bf16)(o[rt][t][r] * inv);
+                }
             }
         }
     }
@@ -429,30 +478,33 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, i
     const int  s = p.row_seq[t], pos = p.row_pos[t];
     const uint64_t* table = p.block_ptrs + (size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    bf16x8 qf[DS];
+    bf16x8 qf[1][DS];
     {
         const __bf16* q = (const __bf16*)p.q + (size_t)t * p.ldq + (size_t)h * D;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
             const int d = ds * 32 + lg * 8;
-            qf[ds]      = (h_ok && d < D) ? *(const bf16x8*)(q + d) : zero8;
+            qf[0][ds]   = (h_ok && d < D) ? *(const bf16x8*)(q + d) : zero8;
         }
     }
-    const float qscale = p.scale * ga_query_temp(p, pos);
+    const float qscale[1] = {p.scale * ga_query_temp(p, pos)};
     const float cap = p.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
-    float   m = -1e30f, l = 0.f;
-    floatx4 o[VT];
+    float   m1[1] = {-1e30f}, l1[1] = {0.f};
+    floatx4 o1[1][VT];
 #pragma unroll
     for (int v = 0; v < VT; ++v) {
-        o[v] = floatx4{0.f, 0.f, 0.f, 0.f};
+        o1[0][v] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
     const int nblk = pos / 64 + 1, per = (nblk + p.splits - 1) / p.splits;
     const int b0 = sp * per, b1 = min(nblk, b0 + per);
     for (int b = b0 + wave; b < b1; b += 4) {
         const char* base = (const char*)table[b] + p.layer_offset;
-        ga_block_step<DS, VT>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D, V,
-                              pos - b * 64, qscale, cap, inv_cap, m, l, o);
+        const int limit[1] = {pos - b * 64};
+        ga_block_step<DS, VT, 1, true>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D,
+                                       V, limit, qscale, cap, inv_cap, m1, l1, o1);
     }
+    const float m = m1[0] * kLn2, l = l1[0];  // back from the log2 domain: the merge below and the split merge kernel use e^x
+    floatx4 (&o)[VT] = o1[0];
     // ---- merge the four waves: common maximum, rescaled sums ----
     if (lg == 0) {
         ml_s[wave][lr][0] = m;
@@ -533,36 +585,44 @@ bool general_attention_tiles_ok(const GeneralAttnParams& p)
            && p.cu_q && p.k_len && p.nseq >= 1 && p.max_q_len >= 1 && p.splits == 1 && p.q_heads % p.kv_heads == 0;
 }
 
-template<int DS>
-static void launch_tiles_ds(const GeneralAttnParams& p, int tiles_per_seq, dim3 grid, hipStream_t st, bool decode)
+// row tiles per wave of the prefill kernel (64 * RT query rows per workgroup): as many as the register file holds without scratch --
+// every key / value fragment a wave loads then serves 16 * RT query rows
+constexpr int tile_rt(int ds, int vt)
 {
-    switch ((p.vdim + 15) / 16) {
+    return (ds <= 4 && vt <= 8) ? 4 : ((ds <= 4 || vt <= 8) ? 2 : 1);
+}
+
+// value sizes are served by the next even tile count (the kernels test channel < vdim), key sizes by 1, 2, 3, 4, 6 or 8 steps
+template<int DS>
+static void launch_tiles_ds(const GeneralAttnParams& p, int arg, dim3 grid, hipStream_t st, bool decode)
+{
+    const int vt = (p.vdim + 15) / 16;
+    switch (vt <= 1 ? 1 : (vt + 1) / 2 * 2) {
 #define TM_TILE_CASE(VT_)                                                           \
     case VT_:                                                                       \
         if (decode) {                                                               \
-            attn_decode_kernel<DS, VT_><<<grid, 256, 0, st>>>(p, tiles_per_seq);    \
+            attn_decode_kernel<DS, VT_><<<grid, 256, 0, st>>>(p, arg);              \
         }                                                                           \
         else {                                                                      \
-            attn_tiles_kernel<DS, VT_><<<grid, 256, 0, st>>>(p, tiles_per_seq);     \
+            attn_tiles_kernel<DS, VT_, tile_rt(DS, VT_)><<<grid, 256, 0, st>>>(p, arg); \
         }                                                                           \
         break;
-        TM_TILE_CASE(1) TM_TILE_CASE(2) TM_TILE_CASE(3) TM_TILE_CASE(4) TM_TILE_CASE(5) TM_TILE_CASE(6) TM_TILE_CASE(7) TM_TILE_CASE(8)
-        TM_TILE_CASE(9) TM_TILE_CASE(10) TM_TILE_CASE(11) TM_TILE_CASE(12) TM_TILE_CASE(13) TM_TILE_CASE(14) TM_TILE_CASE(15) TM_TILE_CASE(16)
+        TM_TILE_CASE(1) TM_TILE_CASE(2) TM_TILE_CASE(4) TM_TILE_CASE(6) TM_TILE_CASE(8) TM_TILE_CASE(10) TM_TILE_CASE(12) TM_TILE_CASE(14)
+        TM_TILE_CASE(16)
 #undef TM_TILE_CASE
     }
 }
 
-static int launch_mfma(const GeneralAttnParams& p, int tiles_per_seq, dim3 grid, hipStream_t st, bool decode)
+static int launch_mfma(const GeneralAttnParams& p, int arg, dim3 grid, hipStream_t st, bool decode)
 {
-    switch ((p.dim + 31) / 32) {
-        case 1: launch_tiles_ds<1>(p, tiles_per_seq, grid, st, decode); break;
-        case 2: launch_tiles_ds<2>(p, tiles_per_seq, grid, st, decode); break;
-        case 3: launch_tiles_ds<3>(p, tiles_per_seq, grid, st, decode); break;
-        case 4: launch_tiles_ds<4>(p, tiles_per_seq, grid, st, decode); break;
-        case 5: launch_tiles_ds<5>(p, tiles_per_seq, grid, st, decode); break;
-        case 6: launch_tiles_ds<6>(p, tiles_per_seq, grid, st, decode); break;
-        case 7: launch_tiles_ds<7>(p, tiles_per_seq, grid, st, decode); break;
-        default: launch_tiles_ds<8>(p, tiles_per_seq, grid, st, decode); break;
+    const int ds = (p.dim + 31) / 32;
+    switch (ds <= 4 ? ds : (ds <= 6 ? 6 : 8)) {
+        case 1: launch_tiles_ds<1>(p, arg, grid, st, decode); break;
+        case 2: launch_tiles_ds<2>(p, arg, grid, st, decode); break;
+        case 3: launch_tiles_ds<3>(p, arg, grid, st, decode); break;
+        case 4: launch_tiles_ds<4>(p, arg, grid, st, decode); break;
+        case 6: launch_tiles_ds<6>(p, arg, grid, st, decode); break;
+        default: launch_tiles_ds<8>(p, arg, grid, st, decode); break;
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;
@@ -595,7 +655,9 @@ int launch_general_attention_tiles(const GeneralAttnParams& p, hipStream_t st)
     if (p.rows == 0) {
         return 0;
     }
-    const int tiles_per_seq = (p.max_q_len + kTileRows - 1) / kTileRows;
+    const int ds = (p.dim + 31) / 32, vt = (p.vdim + 15) / 16;
+    const int rows = kTileRows * tile_rt(ds <= 4 ? ds : (ds <= 6 ? 6 : 8), vt <= 1 ? 1 : (vt + 1) / 2 * 2);  // the instantiation launch_mfma picks
+    const int tiles_per_seq = (p.max_q_len + rows - 1) / rows;
     return launch_mfma(p, tiles_per_seq, dim3(p.nseq * tiles_per_seq, p.q_heads), st, false);
 }
 

@@ -40,16 +40,22 @@ __device__ __forceinline__ void dense_epilogue(void* y, int ldy, int m, int n, f
 }
 
 // ---- bf16, M <= 32 ------------------------------------------------------------------------------------------------------------
-// grid = Np / 16 workgroups of 4 waves.  Wave w covers k-steps w, w + 4, ... (32 k each); MT = 1 or 2 row tiles of 16.
-template<int MT>
+// grid = ceil(N / (16 * NT)) workgroups of 4 waves.  A wave owns NT tiles of 16 output columns x MT tiles of 16 rows and every fourth
+// 128-wide k-chunk (four 32-k MFMA steps: 256 contiguous bytes of every weight row per visit); an activation fragment serves the NT
+// column tiles, a weight fragment the MT row tiles.  The waves' partial sums meet in LDS.
+template<int MT, int NT>
 __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __restrict__ x, int ldx, const __bf16* __restrict__ w, int Kp,
                                                                 void* __restrict__ y, int ldy, int M, int N, int epi, float alpha)
 {
-    __shared__ float red[4][MT][64][4];
+    __shared__ float red[4][MT * NT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n0   = blockIdx.x * 16;
+    const int n0   = blockIdx.x * 16 * NT;
     const int r    = lane & 15, kc = (lane >> 4) * 8;
-    const __bf16* wp = w + (size_t)(n0 + r) * Kp + kc;
+    const __bf16* wp[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        wp[j] = w + (size_t)(n0 + j * 16 + r) * Kp + kc;  // rows up to Np exist (zero): no column test in the loop
+    }
     const __bf16* xp[MT];
     bool          xin[MT];
 #pragma unroll
@@ -57,34 +63,55 @@ __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __
         xin[t] = t * 16 + r < M;
         xp[t]  = x + (size_t)(xin[t] ? t * 16 + r : 0) * ldx + kc;
     }
-    floatx4 acc[MT];
+    floatx4 acc[MT][NT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-        acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            acc[t][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
     }
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll 4
-    for (int k = wave * 32; k < Kp; k += 128) {
-        const bf16x8 b = *(const bf16x8*)(wp + k);
+    for (int k0 = wave * 128; k0 < Kp; k0 += 512) {
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            const bf16x8 a = xin[t] ? *(const bf16x8*)(xp[t] + k) : zero;
-            acc[t]         = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+        for (int kk = 0; kk < 4; ++kk) {
+            const int k = k0 + kk * 32;
+            if (k < Kp) {
+                bf16x8 a[MT], b[NT];
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    b[j] = *(const bf16x8*)(wp[j] + k);
+                }
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    a[t] = xin[t] ? *(const bf16x8*)(xp[t] + k) : zero;
+                }
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+#pragma unroll
+                    for (int j = 0; j < NT; ++j) {
+                        acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], b[j], acc[t][j], 0, 0, 0);
+                    }
+                }
+            }
         }
     }
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            red[wave][t][lane][i] = acc[t][i];
+        for (int j = 0; j < NT; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                red[wave][t * NT + j][lane][i] = acc[t][j][i];
+            }
         }
     }
     __syncthreads();
-    // thread (wave, lane) finishes row tile t = wave % MT ... : 256 threads cover MT * 64 * 4 values, four waves' partials each
-    for (int idx = threadIdx.x; idx < MT * 256; idx += 256) {
-        const int t = idx >> 8, l = (idx >> 2) & 63, i = idx & 3;
-        const float s = (red[0][t][l][i] + red[1][t][l][i]) + (red[2][t][l][i] + red[3][t][l][i]);
-        const int   m = t * 16 + (l >> 4) * 4 + i, n = n0 + (l & 15);  // C fragment: column = lane % 16, rows (lane / 16) * 4 + i
+    for (int idx = threadIdx.x; idx < MT * NT * 256; idx += 256) {
+        const int tj = idx >> 8, l = (idx >> 2) & 63, i = idx & 3;
+        const float s = (red[0][tj][l][i] + red[1][tj][l][i]) + (red[2][tj][l][i] + red[3][tj][l][i]);
+        // C fragment: column = lane % 16, rows (lane / 16) * 4 + i
+        const int m = (tj / NT) * 16 + (l >> 4) * 4 + i, n = n0 + (tj % NT) * 16 + (l & 15);
         if (m < M && n < N) {
             dense_epilogue<__bf16>(y, ldy, m, n, s, epi, alpha);
         }
@@ -286,11 +313,24 @@ int launch_dense_linear(const DenseWeight& d, const void* x, int ldx, void* y, i
     }
     else {
         TM_REQUIRE(ldx % 8 == 0, "dense linear (bf16): rows must be 16-byte aligned");
-        if (M <= 16) {
-            dense_skinny_bf16_kernel<1><<<(d.N + 15) / 16, 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy, M, d.N, epi, alpha);
-        }
-        else if (M <= 32) {
-            dense_skinny_bf16_kernel<2><<<(d.N + 15) / 16, 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy, M, d.N, epi, alpha);
+        if (M <= 32) {
+            // as many column tiles per wave as still leave >= 512 workgroups (two per CU: a workgroup streams its weight rows with a
+            // handful of loads in flight per wave, the device needs many of them): wide outputs amortise the activation reads
+            const int nt = d.N >= 512 * 64 ? 4 : (d.N >= 512 * 32 ? 2 : 1);
+#define TM_SKINNY(MT_, NT_)                                                                                                             \
+    dense_skinny_bf16_kernel<MT_, NT_><<<(d.N + 16 * NT_ - 1) / (16 * NT_), 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, \
+                                                                                        ldy, M, d.N, epi, alpha)
+            if (M <= 16) {
+                if (nt == 4) TM_SKINNY(1, 4);
+                else if (nt == 2) TM_SKINNY(1, 2);
+                else TM_SKINNY(1, 1);
+            }
+            else {
+                if (nt == 4) TM_SKINNY(2, 4);
+                else if (nt == 2) TM_SKINNY(2, 2);
+                else TM_SKINNY(2, 1);
+            }
+#undef TM_SKINNY
         }
         else {
             dense_tiled_bf16_kernel<<<dim3(d.Np / kTN, (M + kTM - 1) / kTM), 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy,
