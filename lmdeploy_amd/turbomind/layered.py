@@ -103,6 +103,11 @@ def _fokonex(c: dict) -> LayeredConfig:
                                 softcap=float(m.get('softcap') or 0.0), qtemp_coef=float(qt.get('coef') or 0.0),
                                 qtemp_every=float(qt.get('every') or 1.0), sink=True, mlp=MLP_DENSE if mlp is not None else MLP_NONE,
                                 ff=int(mlp['ff']) if mlp is not None else 0, act=ACT_RELU2))
+    for s in layers:        # a layer may name a layer that itself runs on another's weights: the tensors are the root's
+        seen = set()
+        while s.weights_of >= 0 and layers[s.weights_of].weights_of >= 0 and s.weights_of not in seen:
+            seen.add(s.weights_of)
+            s.weights_of = layers[s.weights_of].weights_of
     return LayeredConfig(arch='Fokonex', width=int(c['width']), vocab=int(c['vocab']), layers=layers,
                          norm_eps=float(c['norm']['eps']), norm_offset=1.0, residual_mult=float(c['residual_mult']),
                          logit_scale=float(c['logit_scale']), eos_token_id=c.get('eos_token_id'))
