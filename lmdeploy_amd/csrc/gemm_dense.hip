@@ -2,13 +2,14 @@
 //
 //   bf16 : weights and activations bfloat16, fp32 accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16).  Both operands are
 //          K-contiguous, so a lane's MFMA fragment (row = lane % 16, eight consecutive k at (lane / 16) * 8) is ONE 16-byte load.
-//            * skinny kernel (M <= 32, the decode step): a wave owns 16 output columns, the four waves of a workgroup split K and
-//              merge through LDS; weights stream straight from HBM into the fragments, nothing is staged.
+//            * skinny kernel (M <= 32, the decode step): a wave owns 16 or 32 output columns, the four waves of a workgroup split K
+//              and merge through LDS; weights stream straight from HBM into the fragments, one 256-wide chunk ahead of the MFMAs.
 //            * tiled kernel (M > 32, prefill): 128 x 128 x 32 workgroup tiles staged in LDS (padded rows, no bank conflicts on the
 //              16-byte fragment reads), 2 x 2 waves of 64 x 64, next tile prefetched into registers under the MFMAs.
 //   fp32 : true 32-bit FMA arithmetic (no matrix-core shortcut, no reduced-precision mode), 64 x 64 x 16 LDS tiles, 4 x 4 per thread.
 //
-// Weights are kept as zero-padded images [Np][Kp] (Np % 128 == 0, Kp % 32 == 0): no bounds test in any inner loop.  Activation rows
+// Weights are kept as zero-padded images of Np x Kp elements (Np % 128 == 0, Kp % 32 == 0; bf16: in MFMA fragment order, see
+// dense_frag_index; fp32: [Np][Kp]): no bounds test in any inner loop.  Activation rows
 // have a leading dimension >= Kp; what lies in their pad columns only has to be finite, it meets zero weights.
 //
 // The epilogue is chosen per call (DenseEpilogue): plain store, relu(x)^2 (the squared-ReLU feed-forward), accumulate into the fp32
@@ -41,8 +42,12 @@ __device__ __forceinline__ void dense_epilogue(void* y, int ldy, int m, int n, f
 
 // ---- bf16, M <= 32 ------------------------------------------------------------------------------------------------------------
 // grid = ceil(N / (16 * NT)) workgroups of 4 waves.  A wave owns NT tiles of 16 output columns x MT tiles of 16 rows and every fourth
-// 128-wide k-chunk (four 32-k MFMA steps: 256 contiguous bytes of every weight row per visit); an activation fragment serves the NT
-// column tiles, a weight fragment the MT row tiles.  The waves' partial sums meet in LDS.
+// 256-wide k-chunk (eight 32-k MFMA steps: 512 contiguous bytes of every weight row per visit); an activation fragment serves the NT
+// column tiles, a weight fragment the MT row tiles.  The weight stream is what comes from HBM, so it runs one chunk AHEAD in a second
+// register buffer: the loads of chunk c + 1 are in flight under the activation reads (L2 hits) and MFMAs of chunk c.  The waves'
+// partial sums meet in LDS.
+constexpr int kSkinnyKS = 8;  // MFMA steps per chunk
+
 template<int MT, int NT>
 __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __restrict__ x, int ldx, const __bf16* __restrict__ w, int Kp,
                                                                 void* __restrict__ y, int ldy, int M, int N, int epi, float alpha)
@@ -54,7 +59,9 @@ __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __
     const __bf16* wp[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-        wp[j] = w + (size_t)(n0 + j * 16 + r) * Kp + kc;  // rows up to Np exist (zero): no column test in the loop
+        // fragment order: block (tile, k / 32) at ((tile * Kp / 32 + k / 32) * 64 + lane) * 8 -- k advances by 16 elements per k.
+        // Tiles up to Np / 16 exist (zero): no column test in the loop
+        wp[j] = w + ((size_t)(n0 / 16 + j) * (Kp >> 5) * 64 + lane) * 8;
     }
     const __bf16* xp[MT];
     bool          xin[MT];
@@ -72,16 +79,23 @@ __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __
         }
     }
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int k0 = wave * 128; k0 < Kp; k0 += 512) {
+    bf16x8       wa[kSkinnyKS][NT], wb[kSkinnyKS][NT];
+    auto fetch = [&](bf16x8 (&buf)[kSkinnyKS][NT], int k0) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
+        for (int kk = 0; kk < kSkinnyKS; ++kk) {
+            const int k = k0 + kk * 32;
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                buf[kk][j] = k < Kp ? *(const bf16x8*)(wp[j] + (size_t)k * 16) : zero;  // (k / 32) blocks of 512 elements
+            }
+        }
+    };
+    auto compute = [&](const bf16x8 (&buf)[kSkinnyKS][NT], int k0) {
+#pragma unroll
+        for (int kk = 0; kk < kSkinnyKS; ++kk) {
             const int k = k0 + kk * 32;
             if (k < Kp) {
-                bf16x8 a[MT], b[NT];
-#pragma unroll
-                for (int j = 0; j < NT; ++j) {
-                    b[j] = *(const bf16x8*)(wp[j] + k);
-                }
+                bf16x8 a[MT];
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
                     a[t] = xin[t] ? *(const bf16x8*)(xp[t] + k) : zero;
@@ -90,10 +104,28 @@ __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __
                 for (int t = 0; t < MT; ++t) {
 #pragma unroll
                     for (int j = 0; j < NT; ++j) {
-                        acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], b[j], acc[t][j], 0, 0, 0);
+                        acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], buf[kk][j], acc[t][j], 0, 0, 0);
                     }
                 }
             }
+        }
+    };
+    constexpr int kChunk = kSkinnyKS * 32, kStride = 4 * kChunk;  // the four waves interleave their chunks
+    int k0 = wave * kChunk;
+    if (k0 < Kp) {
+        fetch(wa, k0);
+    }
+    for (; k0 < Kp; k0 += 2 * kStride) {
+        const int k1 = k0 + kStride, k2 = k1 + kStride;
+        if (k1 < Kp) {
+            fetch(wb, k1);
+        }
+        compute(wa, k0);
+        if (k2 < Kp) {
+            fetch(wa, k2);
+        }
+        if (k1 < Kp) {
+            compute(wb, k1);
         }
     }
 #pragma unroll
@@ -134,21 +166,24 @@ __global__ __launch_bounds__(256) void dense_tiled_bf16_kernel(const __bf16* __r
     const bool a0 = m0 + sr0 < M, a1 = m0 + sr1 < M;
     const __bf16* ap0 = x + (size_t)(a0 ? m0 + sr0 : 0) * ldx + sk;
     const __bf16* ap1 = x + (size_t)(a1 ? m0 + sr1 : 0) * ldx + sk;
-    const __bf16* bp0 = w + (size_t)(n0 + sr0) * Kp + sk;
-    const __bf16* bp1 = w + (size_t)(n0 + sr1) * Kp + sk;
+    // weights come in fragment order: vector v of a 128 x 32 tile = lane v % 64 of 16-row tile v / 64; it lands in the LDS row of that lane
+    const int bt0 = tid >> 6, bt1 = bt0 + 4, bl = tid & 63;
+    const int br0 = bt0 * 16 + (bl & 15), br1 = bt1 * 16 + (bl & 15), bk = (bl >> 4) * 8;
+    const __bf16* bp0 = w + ((size_t)(n0 / 16 + bt0) * (Kp >> 5) * 64 + bl) * 8;
+    const __bf16* bp1 = w + ((size_t)(n0 / 16 + bt1) * (Kp >> 5) * 64 + bl) * 8;
     const bf16x8  zero = {0, 0, 0, 0, 0, 0, 0, 0};
     bf16x8        ra0, ra1, rb0, rb1;
     auto fetch = [&](int k) {
         ra0 = a0 ? *(const bf16x8*)(ap0 + k) : zero;
         ra1 = a1 ? *(const bf16x8*)(ap1 + k) : zero;
-        rb0 = *(const bf16x8*)(bp0 + k);
-        rb1 = *(const bf16x8*)(bp1 + k);
+        rb0 = *(const bf16x8*)(bp0 + (size_t)k * 16);
+        rb1 = *(const bf16x8*)(bp1 + (size_t)k * 16);
     };
     auto stash = [&](int buf) {
         *(bf16x8*)(&sa[buf][sr0 * kLdsRow + sk]) = ra0;
         *(bf16x8*)(&sa[buf][sr1 * kLdsRow + sk]) = ra1;
-        *(bf16x8*)(&sb[buf][sr0 * kLdsRow + sk]) = rb0;
-        *(bf16x8*)(&sb[buf][sr1 * kLdsRow + sk]) = rb1;
+        *(bf16x8*)(&sb[buf][br0 * kLdsRow + bk]) = rb0;
+        *(bf16x8*)(&sb[buf][br1 * kLdsRow + bk]) = rb1;
     };
     floatx4 acc[4][4];
 #pragma unroll
@@ -254,13 +289,26 @@ __global__ __launch_bounds__(256) void dense_f32_kernel(const float* __restrict_
 
 // ---- weight images ----------------------------------------------------------------------------------------------------------------
 // src: bf16 [rows][cols] (checkpoint bytes) -> dst[(row0 + r) * Kp + col0 + c], T = bf16 (copy) or float (exact widening)
+// bf16 images are stored in FRAGMENT ORDER: the 16 rows x 32 k block (n / 16, k / 32) is one contiguous KB laid out as the 64 lanes of
+// its MFMA fragment (lane = (k % 32) / 8 * 16 + n % 16, eight k each), blocks of one 16-row tile consecutive along k -- a wave's fragment
+// load is one contiguous KB and a workgroup streams whole contiguous runs of HBM instead of 64-byte pieces of 16 rows
+__host__ __device__ inline size_t dense_frag_index(int n, int k, int Kp)
+{
+    return ((((size_t)(n >> 4) * (Kp >> 5) + (k >> 5)) * 64 + ((k & 31) >> 3) * 16 + (n & 15)) << 3) + (k & 7);
+}
+
 template<class T>
 __global__ void dense_place_kernel(T* __restrict__ dst, int Kp, int row0, int col0, const __bf16* __restrict__ src, int rows, int cols)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < (size_t)rows * cols) {
         const int r = (int)(i / cols), c = (int)(i % cols);
-        dst[(size_t)(row0 + r) * Kp + col0 + c] = (T)(float)src[i];
+        if constexpr (sizeof(T) == 2) {
+            dst[dense_frag_index(row0 + r, col0 + c, Kp)] = (T)(float)src[i];
+        }
+        else {
+            dst[(size_t)(row0 + r) * Kp + col0 + c] = (T)(float)src[i];
+        }
     }
 }
 
@@ -314,20 +362,17 @@ int launch_dense_linear(const DenseWeight& d, const void* x, int ldx, void* y, i
     else {
         TM_REQUIRE(ldx % 8 == 0, "dense linear (bf16): rows must be 16-byte aligned");
         if (M <= 32) {
-            // as many column tiles per wave as still leave >= 512 workgroups (two per CU: a workgroup streams its weight rows with a
-            // handful of loads in flight per wave, the device needs many of them): wide outputs amortise the activation reads
-            const int nt = d.N >= 512 * 64 ? 4 : (d.N >= 512 * 32 ? 2 : 1);
+            // two column tiles per wave where that still leaves >= 512 workgroups (two per CU): wide outputs amortise the activation reads
+            const int nt = d.N >= 512 * 32 ? 2 : 1;
 #define TM_SKINNY(MT_, NT_)                                                                                                             \
     dense_skinny_bf16_kernel<MT_, NT_><<<(d.N + 16 * NT_ - 1) / (16 * NT_), 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, \
                                                                                         ldy, M, d.N, epi, alpha)
             if (M <= 16) {
-                if (nt == 4) TM_SKINNY(1, 4);
-                else if (nt == 2) TM_SKINNY(1, 2);
+                if (nt == 2) TM_SKINNY(1, 2);
                 else TM_SKINNY(1, 1);
             }
             else {
-                if (nt == 4) TM_SKINNY(2, 4);
-                else if (nt == 2) TM_SKINNY(2, 2);
+                if (nt == 2) TM_SKINNY(2, 2);
                 else TM_SKINNY(2, 1);
             }
 #undef TM_SKINNY
