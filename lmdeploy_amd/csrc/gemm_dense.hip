@@ -42,11 +42,10 @@ __device__ __forceinline__ void dense_epilogue(void* y, int ldy, int m, int n, f
 
 // ---- bf16, M <= 32 ------------------------------------------------------------------------------------------------------------
 // grid = ceil(N / (16 * NT)) workgroups of 4 waves.  A wave owns NT tiles of 16 output columns x MT tiles of 16 rows and every fourth
-// 256-wide k-chunk (eight 32-k MFMA steps: 512 contiguous bytes of every weight row per visit); an activation fragment serves the NT
+// k-chunk (eight 32-k MFMA steps with one column tile, four with two); an activation fragment serves the NT
 // column tiles, a weight fragment the MT row tiles.  The weight stream is what comes from HBM, so it runs one chunk AHEAD in a second
 // register buffer: the loads of chunk c + 1 are in flight under the activation reads (L2 hits) and MFMAs of chunk c.  The waves'
 // partial sums meet in LDS.
-constexpr int kSkinnyKS = 8;  // MFMA steps per chunk
 
 template<int MT, int NT>
 __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __restrict__ x, int ldx, const __bf16* __restrict__ w, int Kp,
@@ -78,6 +77,8 @@ __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __
             acc[t][j] = floatx4{0.f, 0.f, 0.f, 0.f};
         }
     }
+    // MFMA steps per chunk: two chunk buffers of KS x NT fragments must leave room for three to four waves per SIMD
+    constexpr int kSkinnyKS = NT == 1 ? 8 : 4;
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
     bf16x8       wa[kSkinnyKS][NT], wb[kSkinnyKS][NT];
     auto fetch = [&](bf16x8 (&buf)[kSkinnyKS][NT], int k0) {

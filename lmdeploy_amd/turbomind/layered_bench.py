@@ -25,7 +25,7 @@ SIZES = {
 def _fokonex_engine(s, batch, session_len, max_prefill):
     from . import layered
     spec = layered.LayerSpec(heads=s['heads'], kv_heads=s['kv_heads'], dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0, qtemp_coef=0.1,
-                             qtemp_every=256.0, sink=True, mlp=layered.MLP_DENSE, ff=s['inter'] * 3 // 2)
+                             qtemp_every=512.0, sink=True, mlp=layered.MLP_DENSE, ff=s['inter'] * 3 // 2)
     cfg = layered.LayeredConfig('Fokonex', s['width'], s['vocab'], [spec] * s['layers'], 1e-5, 1.0, 0.5, 1.0)
     eng = layered.LayeredEngine(cfg, dtype='bfloat16', max_batch_size=batch, session_len=session_len, max_prefill_token_num=max_prefill)
     eng.init_synthetic(seed=1)

@@ -149,7 +149,7 @@ SPECS = {
     'cap': dict(heads=4, kv_heads=2, dim=32, vdim=16, scale=0.9, softcap=3.0, qtemp_coef=0.0, qtemp_every=1.0),
     'temp': dict(heads=4, kv_heads=2, dim=32, vdim=16, scale=0.2, softcap=0.0, qtemp_coef=0.7, qtemp_every=3.0),
     'all_odd': dict(heads=6, kv_heads=2, dim=40, vdim=24, scale=0.15, softcap=8.0, qtemp_coef=0.4, qtemp_every=64.0),
-    'one_group': dict(heads=3, kv_heads=3, dim=72, vdim=136, scale=0.1, softcap=30.0, qtemp_coef=0.3, qtemp_every=100.0),
+    'one_group': dict(heads=3, kv_heads=3, dim=72, vdim=136, scale=0.1, softcap=30.0, qtemp_coef=0.25, qtemp_every=100.0),
     'unaligned': dict(heads=2, kv_heads=1, dim=20, vdim=12, scale=0.2, softcap=5.0, qtemp_coef=0.1, qtemp_every=7.0),
 }
 
@@ -212,7 +212,7 @@ def test_attention_finds_one_far_key_and_respects_the_causal_edge(tm, cuda, dtyp
 
 
 @pytest.mark.parametrize('dtype', [0, 1])
-@pytest.mark.parametrize('heads,kv_heads,D,V', [(4, 4, 32, 16), (6, 2, 40, 24), (40, 2, 64, 48), (8, 1, 128, 128), (2, 1, 20, 12)])
+@pytest.mark.parametrize('heads,kv_heads,D,V', [(4, 4, 32, 16), (6, 2, 40, 24), (40, 2, 72, 40), (8, 1, 128, 128), (2, 1, 20, 12)])
 def test_attention_decode_rows_of_unequal_sequences(tm, cuda, dtype, heads, kv_heads, D, V):
     """one new row per sequence, contexts from 1 token to several blocks (one ends exactly at a block border, one just behind it): the
     row kernel with and without key splits, and in bf16 the matrix-core decode kernel (query heads as rows: groups of 1, 3, 8 and 20)"""
@@ -241,7 +241,7 @@ def test_attention_decode_rows_of_unequal_sequences(tm, cuda, dtype, heads, kv_h
 
 # ---- engine -------------------------------------------------------------------------------------------------------------------------
 def _layer(**kw):
-    d = dict(heads=4, kv_heads=2, dim=40, vdim=24, scale=0.16, softcap=9.0, qtemp_coef=0.3, qtemp_every=7, sink=True, ff=136, weights_of=-1)
+    d = dict(heads=4, kv_heads=2, dim=40, vdim=24, scale=0.16, softcap=9.0, qtemp_coef=0.35, qtemp_every=7, sink=True, ff=136, weights_of=-1)
     d.update(kw)
     return d
 
