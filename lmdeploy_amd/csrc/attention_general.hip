@@ -280,7 +280,7 @@ __device__ __forceinline__ float ga_tanh_fast(float x)
 // Every key / value fragment is loaded ONCE and serves all RT row tiles; the value fragments are requested before the soft-max
 // arithmetic so that their latency hides under it.  qf: the rows' query fragments; limit: last visible key of the lane's rows
 // (block-relative; < 0: none); kb / vb: the key head's keys [64][D] and transposed values [V][64] of this block.
-template<int DS, int VT, int RT, bool MASK>
+template<int DS, int VT, int RT, bool MASK, bool EAGER>
 __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const __bf16* __restrict__ kb, const __bf16* __restrict__ vb, int D,
                                               int V, const int (&limit)[RT], const float (&qscale)[RT], float cap, float inv_cap,
                                               float (&m)[RT], float (&l)[RT], floatx4 (&o)[RT][VT])
@@ -297,8 +297,18 @@ __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const 
         const __bf16* kr = kb + (size_t)((kt >> 1) * 32 + (lr >> 2) * 8 + (kt & 1) * 4 + (lr & 3)) * D;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
-            const int    d  = ds * 32 + lg * 8;
-            const bf16x8 kf = d < D ? *(const bf16x8*)(kr + d) : zero8;
+            // EAGER (decode: a wave has one or two blocks, latency is everything): every load is unconditional -- clamped address, value
+            // selected afterwards -- so that all of them are in flight at once; a guarded load is waited for at the join of its branch.
+            // The prefill kernel keeps the guarded form: with four row tiles per wave the eager form costs registers it does not have.
+            const int d = ds * 32 + lg * 8;
+            bf16x8    kf;
+            if constexpr (EAGER) {
+                const bf16x8 kl = *(const bf16x8*)(kr + min(d, D - 8));
+                kf              = d < D ? kl : zero8;
+            }
+            else {
+                kf = d < D ? *(const bf16x8*)(kr + d) : zero8;
+            }
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 sc[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[rt][ds], sc[rt][kt], 0, 0, 0);
@@ -308,10 +318,18 @@ __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const 
     bf16x8 vf[VT][2];
 #pragma unroll
     for (int t = 0; t < VT; ++t) {
-        const int     v  = t * 16 + lr;
-        const __bf16* vr = vb + (size_t)v * 64 + lg * 8;
-        vf[t][0]         = v < V ? *(const bf16x8*)(vr) : zero8;
-        vf[t][1]         = v < V ? *(const bf16x8*)(vr + 32) : zero8;
+        const int v = t * 16 + lr;
+        if constexpr (EAGER) {
+            const __bf16* vr = vb + (size_t)min(v, V - 1) * 64 + lg * 8;
+            const bf16x8  v0 = *(const bf16x8*)(vr), v1 = *(const bf16x8*)(vr + 32);
+            vf[t][0]         = v < V ? v0 : zero8;
+            vf[t][1]         = v < V ? v1 : zero8;
+        }
+        else {
+            const __bf16* vr = vb + (size_t)v * 64 + lg * 8;
+            vf[t][0]         = v < V ? *(const bf16x8*)(vr) : zero8;
+            vf[t][1]         = v < V ? *(const bf16x8*)(vr + 32) : zero8;
+        }
     }
     // lane holds S[row lr of tile rt][key (kt / 2) * 32 + lg * 8 + (kt % 2) * 4 + r].  From here on scores live in the log2 domain
     // (multiplied by log2 e) so that every exponential is one v_exp_f32: the capped score is
@@ -405,8 +423,9 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
         const __bf16* q = (const __bf16*)p.q + (size_t)(row_base + (q_ok[rt] ? qi : 0)) * p.ldq + (size_t)h * D;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
-            const int d = ds * 32 + lg * 8;
-            qf[rt][ds]  = (q_ok[rt] && d < D) ? *(const bf16x8*)(q + d) : zero8;
+            const int    d  = ds * 32 + lg * 8;
+            const bf16x8 ql = *(const bf16x8*)(q + min(d, D - 8));
+            qf[rt][ds]      = (q_ok[rt] && d < D) ? ql : zero8;
         }
         qscale[rt] = p.scale * ga_query_temp(p, pos[rt]);
         m[rt]      = -1e30f;
@@ -427,10 +446,10 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
         }
         const __bf16 *kb = (const __bf16*)base + (size_t)g * 64 * D, *vb = (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V;
         if (b * 64 + 63 <= pos0 + row0) {  // every row of the wave sees the whole block (rows beyond the portion are discarded anyway)
-            ga_block_step<DS, VT, RT, false>(qf, kb, vb, D, V, limit, qscale, cap, inv_cap, m, l, o);
+            ga_block_step<DS, VT, RT, false, false>(qf, kb, vb, D, V, limit, qscale, cap, inv_cap, m, l, o);
         }
         else {
-            ga_block_step<DS, VT, RT, true>(qf, kb, vb, D, V, limit, qscale, cap, inv_cap, m, l, o);
+            ga_block_step<DS, VT, RT, true, false>(qf, kb, vb, D, V, limit, qscale, cap, inv_cap, m, l, o);
         }
     }
 #pragma unroll
@@ -483,8 +502,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, i
         const __bf16* q = (const __bf16*)p.q + (size_t)t * p.ldq + (size_t)h * D;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
-            const int d = ds * 32 + lg * 8;
-            qf[0][ds]   = (h_ok && d < D) ? *(const bf16x8*)(q + d) : zero8;
+            const int    d  = ds * 32 + lg * 8;
+            const bf16x8 ql = *(const bf16x8*)(q + min(d, D - 8));
+            qf[0][ds]       = (h_ok && d < D) ? ql : zero8;
         }
     }
     const float qscale[1] = {p.scale * ga_query_temp(p, pos)};
@@ -500,7 +520,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, i
     for (int b = b0 + wave; b < b1; b += 4) {
         const char* base = (const char*)table[b] + p.layer_offset;
         const int limit[1] = {pos - b * 64};
-        ga_block_step<DS, VT, 1, true>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D,
+        ga_block_step<DS, VT, 1, true, true>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D,
                                        V, limit, qscale, cap, inv_cap, m1, l1, o1);
     }
     const float m = m1[0] * kLn2, l = l1[0];  // back from the log2 domain: the merge below and the split merge kernel use e^x

@@ -41,17 +41,18 @@ __device__ __forceinline__ void dense_epilogue(void* y, int ldy, int m, int n, f
 }
 
 // ---- bf16, M <= 32 ------------------------------------------------------------------------------------------------------------
-// grid = ceil(N / (16 * NT)) workgroups of 4 waves.  A wave owns NT tiles of 16 output columns x MT tiles of 16 rows and every fourth
+// grid = ceil(N / (16 * NT)) workgroups of 4, 8 or 16 waves (narrow outputs with a long K: more waves split K so that the device still
+// holds enough of them to cover the HBM latency).  A wave owns NT tiles of 16 output columns x MT tiles of 16 rows and every fourth
 // k-chunk (eight 32-k MFMA steps with one column tile, four with two); an activation fragment serves the NT
 // column tiles, a weight fragment the MT row tiles.  The weight stream is what comes from HBM, so it runs one chunk AHEAD in a second
 // register buffer: the loads of chunk c + 1 are in flight under the activation reads (L2 hits) and MFMAs of chunk c.  The waves'
 // partial sums meet in LDS.
 
-template<int MT, int NT>
-__global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __restrict__ x, int ldx, const __bf16* __restrict__ w, int Kp,
+template<int MT, int NT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void dense_skinny_bf16_kernel(const __bf16* __restrict__ x, int ldx, const __bf16* __restrict__ w, int Kp,
                                                                 void* __restrict__ y, int ldy, int M, int N, int epi, float alpha)
 {
-    __shared__ float red[4][MT * NT][64][4];
+    __shared__ float red[WAVES][MT * NT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0   = blockIdx.x * 16 * NT;
     const int r    = lane & 15, kc = (lane >> 4) * 8;
@@ -87,7 +88,8 @@ __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __
             const int k = k0 + kk * 32;
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
-                buf[kk][j] = k < Kp ? *(const bf16x8*)(wp[j] + (size_t)k * 16) : zero;  // (k / 32) blocks of 512 elements
+                const bf16x8 v = *(const bf16x8*)(wp[j] + (size_t)min(k, Kp - 32) * 16);  // (k / 32) blocks of 512 elements; loads are
+                buf[kk][j]     = k < Kp ? v : zero;                                        // unconditional so that all stay in flight
             }
         }
     };
@@ -99,7 +101,8 @@ __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __
                 bf16x8 a[MT];
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
-                    a[t] = xin[t] ? *(const bf16x8*)(xp[t] + k) : zero;
+                    const bf16x8 v = *(const bf16x8*)(xp[t] + k);  // (rows beyond M read row 0)
+                    a[t]           = xin[t] ? v : zero;
                 }
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
@@ -111,7 +114,7 @@ __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __
             }
         }
     };
-    constexpr int kChunk = kSkinnyKS * 32, kStride = 4 * kChunk;  // the four waves interleave their chunks
+    constexpr int kChunk = kSkinnyKS * 32, kStride = WAVES * kChunk;  // the waves interleave their chunks
     int k0 = wave * kChunk;
     if (k0 < Kp) {
         fetch(wa, k0);
@@ -140,9 +143,13 @@ __global__ __launch_bounds__(256) void dense_skinny_bf16_kernel(const __bf16* __
         }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < MT * NT * 256; idx += 256) {
+    for (int idx = threadIdx.x; idx < MT * NT * 256; idx += WAVES * 64) {
         const int tj = idx >> 8, l = (idx >> 2) & 63, i = idx & 3;
-        const float s = (red[0][tj][l][i] + red[1][tj][l][i]) + (red[2][tj][l][i] + red[3][tj][l][i]);
+        float     s  = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < WAVES; wv += 4) {  // fixed order: the result does not depend on which wave finished first
+            s += (red[wv][tj][l][i] + red[wv + 1][tj][l][i]) + (red[wv + 2][tj][l][i] + red[wv + 3][tj][l][i]);
+        }
         // C fragment: column = lane % 16, rows (lane / 16) * 4 + i
         const int m = (tj / NT) * 16 + (l >> 4) * 4 + i, n = n0 + (tj % NT) * 16 + (l & 15);
         if (m < M && n < N) {
@@ -175,8 +182,9 @@ __global__ __launch_bounds__(256) void dense_tiled_bf16_kernel(const __bf16* __r
     const bf16x8  zero = {0, 0, 0, 0, 0, 0, 0, 0};
     bf16x8        ra0, ra1, rb0, rb1;
     auto fetch = [&](int k) {
-        ra0 = a0 ? *(const bf16x8*)(ap0 + k) : zero;
-        ra1 = a1 ? *(const bf16x8*)(ap1 + k) : zero;
+        const bf16x8 v0 = *(const bf16x8*)(ap0 + k), v1 = *(const bf16x8*)(ap1 + k);  // unconditional (rows beyond M read row 0)
+        ra0 = a0 ? v0 : zero;
+        ra1 = a1 ? v1 : zero;
         rb0 = *(const bf16x8*)(bp0 + (size_t)k * 16);
         rb1 = *(const bf16x8*)(bp1 + (size_t)k * 16);
     };
@@ -364,18 +372,42 @@ int launch_dense_linear(const DenseWeight& d, const void* x, int ldx, void* y, i
         TM_REQUIRE(ldx % 8 == 0, "dense linear (bf16): rows must be 16-byte aligned");
         if (M <= 32) {
             // two column tiles per wave where that still leaves >= 512 workgroups (two per CU): wide outputs amortise the activation reads
-            const int nt = d.N >= 512 * 32 ? 2 : 1;
-#define TM_SKINNY(MT_, NT_)                                                                                                             \
-    dense_skinny_bf16_kernel<MT_, NT_><<<(d.N + 16 * NT_ - 1) / (16 * NT_), 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, \
-                                                                                        ldy, M, d.N, epi, alpha)
+            const int nt     = d.N >= 512 * 32 ? 2 : 1;
+            const int wgs    = (d.N + 16 * nt - 1) / (16 * nt);
+            const int chunk  = (nt == 1 ? 8 : 4) * 32;
+            int       waves  = 4;  // ... and more waves per workgroup while the device holds fewer than 16 per CU and K has a chunk for each
+            while (waves < (nt == 1 ? 16 : 8) && wgs * waves < 256 * 16 && d.Kp >= chunk * 2 * waves) {
+                waves *= 2;
+            }
+#define TM_SKINNY(MT_, NT_, W_)                                                                                                     \
+    dense_skinny_bf16_kernel<MT_, NT_, W_><<<wgs, W_ * 64, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy, M, d.N, epi, alpha)
+#define TM_SKINNY_W(MT_, NT_)                     \
+    if (waves == 16 && NT_ == 1) {                \
+        TM_SKINNY(MT_, 1, 16);                    \
+    }                                             \
+    else if (waves >= 8) {                        \
+        TM_SKINNY(MT_, NT_, 8);                   \
+    }                                             \
+    else {                                        \
+        TM_SKINNY(MT_, NT_, 4);                   \
+    }
             if (M <= 16) {
-                if (nt == 2) TM_SKINNY(1, 2);
-                else TM_SKINNY(1, 1);
+                if (nt == 2) {
+                    TM_SKINNY_W(1, 2)
+                }
+                else {
+                    TM_SKINNY_W(1, 1)
+                }
             }
             else {
-                if (nt == 2) TM_SKINNY(2, 2);
-                else TM_SKINNY(2, 1);
+                if (nt == 2) {
+                    TM_SKINNY_W(2, 2)
+                }
+                else {
+                    TM_SKINNY_W(2, 1)
+                }
             }
+#undef TM_SKINNY_W
 #undef TM_SKINNY
         }
         else {
