@@ -189,7 +189,7 @@ int layered_start(tm_engine* e)
     e->max_blocks_per_seq = (c.session_len + c.cache_block_seq_len - 1) / c.cache_block_seq_len;
     e->max_tokens         = std::max(B, std::max(64, c.max_prefill_token_num));
     const size_t T        = e->max_tokens;
-    // cache block: every layer's keys [kv_heads][block_len][dim] and values [kv_heads][block_len][vdim]
+    // cache block: every layer run has its keys [kv_heads][block_len][dim] and, behind them, its values transposed [kv_heads][vdim][block_len]
     int64_t off = 0;
     int     max_qkv = 0, max_cat = 0, max_vdim = 0, max_heads = 0;
     for (LmLayer& L : lm.layers) {
