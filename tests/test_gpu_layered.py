@@ -3,7 +3,11 @@
 decoding, portions, unequal batches, reused blocks and slots, long decoding, and greedy generation through the static batch, the
 scheduler and the pipeline.  Configurations and weights are the tests' own."""
 import ctypes as C
+import json
 import math
+import os
+import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -421,3 +425,50 @@ def test_pipeline_serves_a_checkpoint_folder(cuda, tmp_path):
         sampled = pipe(prompts, gen_config=GenerationConfig(max_new_tokens=6, ignore_eos=True, do_sample=True, top_k=5, temperature=0.8,
                                                             random_seed=11))
         assert all(len(r.token_ids) == 6 and all(0 <= t < cfg['vocab'] for t in r.token_ids) for r in sampled)
+
+
+def test_trace_run_replays_a_schedule_on_awkward_sizes(cuda, tmp_path):
+    """bin/trace_run end to end, both number formats: a checkpoint folder with a width off the 8 grid, key / value sizes off it too, a group of
+    17 query heads per key head, a non-integer temperature period, a layer without cap and temperature keys, weight sharing through a chain;
+    five requests in shared steps, pool of 640 tokens"""
+    def L(**kw):
+        d = dict(heads=5, kv_heads=1, dim=24, vdim=40, scale=0.21, softcap=11.0, qtemp_coef=0.45, qtemp_every=33, sink=True, ff=72, weights_of=-1)
+        d.update(kw)
+        return d
+    B = dict(heads=6, kv_heads=3, dim=20, vdim=12, ff=0, softcap=0.0, qtemp_coef=0.0)
+    Cc = dict(heads=34, kv_heads=2, dim=8, vdim=8, ff=200, qtemp_every=2.5)
+    cfg = lo.make_config(100, 333, [L(), L(**B), L(weights_of=0), L(weights_of=1, **B), L(**Cc), L(weights_of=4, **Cc), L(weights_of=0)], mult=0.2,
+                         logit_scale=3.0)
+    w = lo.make_weights(cfg, 11)
+    folder = str(tmp_path / 'model')
+    lo.write_checkpoint(folder, cfg, w)
+    c = json.load(open(folder + '/config.json'))
+    c['layers'][6]['weights_of'] = 2                      # a chain: 6 -> 2 -> 0
+    del c['layers'][1]['mixer']['q_temp'], c['layers'][1]['mixer']['softcap']
+    json.dump(c, open(folder + '/config.json', 'w'))
+    rng = np.random.default_rng(0)
+    reqs = {n: rng.integers(0, 333, k).tolist() for n, k in (('a', 300), ('b', 70), ('c', 1), ('d', 129), ('e', 40))}
+    ref = {n: lo.forward(cfg, w, t)[0] for n, t in reqs.items()}
+    plan = [[('a', 100)], [('a', 3), ('b', 64), ('c', 1)], [('a', 1), ('b', 2), ('d', 65)], [('a', 64), ('b', 1), ('d', 1), ('e', 2)],
+            [('a', 2), ('b', 3), ('d', 63), ('e', 38)], [('a', 130)]]
+    at, steps, rows = {n: 0 for n in reqs}, [], []
+    for i, st_ in enumerate(plan):
+        ent, end, rr = [], [], []
+        for n, k in st_:
+            ent.append({'id': n, 'tokens': reqs[n][at[n]:at[n] + k], 'want': list(range(0, k, 2))})
+            rr += [(n, at[n] + j) for j in range(0, k, 2)]
+            at[n] += k
+            if at[n] == len(reqs[n]):
+                end.append(n)
+        steps.append(json.dumps({'step': i, 'entries': ent, 'end': end}))
+        rows.append(rr)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for dtype, tol in (('float32', 5e-5), ('bfloat16', 5e-2)):
+        out = str(tmp_path / dtype)
+        p = subprocess.run([sys.executable, os.path.join(root, 'bin', 'trace_run'), '--model', folder, '--dtype', dtype, '--out', out,
+                            '--max-tokens', '640'], input='\n'.join(steps) + '\n', text=True, capture_output=True, timeout=100)
+        assert p.returncode == 0, p.stderr[-2000:]
+        assert [l for l in p.stdout.split('\n') if l.startswith('done')] == ['done %d' % i for i in range(len(plan))]
+        for i, rr in enumerate(rows):
+            got = np.fromfile(os.path.join(out, '%d.f32' % i), '<f4').reshape(len(rr), -1)
+            assert rel_err(got, np.stack([ref[n][j] for n, j in rr])) <= tol, (dtype, i)
