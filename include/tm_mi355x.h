@@ -505,10 +505,28 @@ int tm_gemm_export(const char* path);
  * Norms, attention scores and weights, and the residual sum are fp32 in both.
  * Weight slots (tm_engine_weight_copy, checkpoint bytes: bf16, [out][in]): "embed", "l<i>.norm1", "l<i>.norm2" (with an ff),
  * "l<i>.mix.q|k|v|o", "l<i>.mix.sink" (with a sink), "l<i>.mlp.up|down", "final.norm", "head". */
-enum { TM_MIXER_ATTENTION = 1 };
-enum { TM_MLP_NONE = 0, TM_MLP_DENSE = 1 };
-enum { TM_ACT_RELU2 = 0 };
+enum { TM_MIXER_ATTENTION = 1, TM_MIXER_LATENT = 2 };
+enum { TM_MLP_NONE = 0, TM_MLP_DENSE = 1, TM_MLP_GATED = 2, TM_MLP_MOE = 3 };
+enum { TM_ACT_RELU2 = 0, TM_ACT_GELU_TANH = 1, TM_ACT_SILU = 2 };
 enum { TM_DTYPE_BF16 = 0, TM_DTYPE_F32 = 1 };
+/* Further block forms, mixers and feed-forwards (every switch off at 0: the block above):
+ *   one_norm:    both sublayers read norm1(x) (no norm2)
+ *   resid_gate:  x <- x + sigmoid(rg1 h + rg1.b) * mixer(h) + sigmoid(rg2 h + rg2.b) * ff(h), element by element, h = the sublayers' input
+ *                (slots "l<i>.rg1", "l<i>.rg1.b", and "l<i>.rg2", "l<i>.rg2.b" with an ff)
+ *   loop_pass:   >= 0: this layer run opens pass `loop_pass` of a loop: before it x <- loop.in [x; x0] + loop.step[loop_pass], x0 the
+ *                embedding output (slots "loop.in" [width][2 width], "loop.step" [loop_times][width]); the runs of later passes name the
+ *                first pass's layers in weights_of
+ *   attention:   qk_unit_norm / v_unit_norm: queries and keys / values are scaled to root mean square 1 per head (no weight, norm_eps);
+ *                dist_bias: score -= r1[head] * ln(1 + r2[head] * (i - j)) ("mix.r1", "mix.r2"); chunk > 0: position i sees j <= i only
+ *                inside its own chunk, floor(i / chunk) = floor(j / chunk); out_gate: head h's output *= sigmoid(g h)[h] ("mix.g" [heads][width])
+ *   TM_MIXER_LATENT: per token one latent vector c = norm(dkv h [0, kv_rank)) * "mix.dkv.norm" and one rotated key part
+ *                rot(dkv h [kv_rank, kv_rank + rot_dim)) shared by all heads are cached; head a: key = [uk_a c | rotated part], value = uv_a c,
+ *                query = [q_a h [0, dim) | rot(q_a h [dim, dim + rot_dim))]; rotation pairs channel i with i + rot_dim / 2, angle =
+ *                position * rot_base^(-2 i / rot_dim); causal; sink as above.  kv_heads = 1.  Slots "mix.q" [heads (dim + rot_dim)][width],
+ *                "mix.dkv" [kv_rank + rot_dim][width], "mix.dkv.norm", "mix.uk" [heads dim][kv_rank], "mix.uv" [heads vdim][kv_rank], "mix.o"
+ *   TM_MLP_GATED: down(act(gate h) * (up h)) ("mlp.gate", "mlp.up", "mlp.down"); act TM_ACT_GELU_TANH | TM_ACT_SILU | TM_ACT_RELU2
+ *   TM_MLP_MOE:  `experts` gated feed-forwards of size ff ("mlp.e<j>.gate|up|down"), router scores sigmoid("mlp.router" h) in fp32, the
+ *                `top` largest win, their scores (not renormalised) multiply the expert's INPUT: sum_e expert_e(score_e * h) */
 typedef struct tm_layer_spec {
     int   mixer;
     int   weights_of; /* -1: own tensors */
@@ -516,12 +534,18 @@ typedef struct tm_layer_spec {
     float scale, softcap, qtemp_coef, qtemp_every;
     int   sink;
     int   mlp, ff, act;
+    int   one_norm, resid_gate, loop_pass;
+    int   qk_unit_norm, v_unit_norm, dist_bias, out_gate, chunk;
+    int   kv_rank, rot_dim;
+    float rot_base;
+    int   experts, top;
 } tm_layer_spec;
 typedef struct tm_layered_config {
     int                  width, vocab, n_layers;
     const tm_layer_spec* layers;
     float                norm_eps, norm_offset, residual_mult, logit_scale;
     int                  dtype;
+    int                  loop_times; /* 0: no loop tensors */
 } tm_layered_config;
 /* cfg->model is ignored; tp must be 1; quant_policy 0 (the cache holds the activation type) */
 int tm_engine_create_layered(tm_engine** out, const tm_engine_config* cfg, const tm_layered_config* model);

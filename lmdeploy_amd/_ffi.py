@@ -71,13 +71,15 @@ class LayerSpec(C.Structure):
     """struct tm_layer_spec"""
     _fields_ = [('mixer', c_int), ('weights_of', c_int), ('heads', c_int), ('kv_heads', c_int), ('dim', c_int), ('vdim', c_int),
                 ('scale', c_float), ('softcap', c_float), ('qtemp_coef', c_float), ('qtemp_every', c_float), ('sink', c_int),
-                ('mlp', c_int), ('ff', c_int), ('act', c_int)]
+                ('mlp', c_int), ('ff', c_int), ('act', c_int), ('one_norm', c_int), ('resid_gate', c_int), ('loop_pass', c_int),
+                ('qk_unit_norm', c_int), ('v_unit_norm', c_int), ('dist_bias', c_int), ('out_gate', c_int), ('chunk', c_int),
+                ('kv_rank', c_int), ('rot_dim', c_int), ('rot_base', c_float), ('experts', c_int), ('top', c_int)]
 
 
 class LayeredConfig(C.Structure):
     """struct tm_layered_config"""
     _fields_ = [('width', c_int), ('vocab', c_int), ('n_layers', c_int), ('layers', POINTER(LayerSpec)), ('norm_eps', c_float),
-                ('norm_offset', c_float), ('residual_mult', c_float), ('logit_scale', c_float), ('dtype', c_int)]
+                ('norm_offset', c_float), ('residual_mult', c_float), ('logit_scale', c_float), ('dtype', c_int), ('loop_times', c_int)]
 
 
 class StepEntry(C.Structure):

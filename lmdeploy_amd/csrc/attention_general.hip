@@ -4,6 +4,10 @@
 //   * soft cap:                      score  = cap * tanh(score / cap)                               (cap <= 0: off)
 //   * attention sink:                the softmax denominator also holds exp(sink[head]): a learned logit with no key and no value,
 //                                    neither scaled nor capped                                      (sink = nullptr: off)
+//   * distance penalty:              score -= r1[head] * ln(1 + r2[head] * (p - key position))      (dist_r1 = nullptr: off)
+//   * chunked visibility:            a row sees the keys of its own chunk of positions only:
+//                                    key >= floor(p / chunk) * chunk, chunks counted from position 0   (chunk = 0: off)
+//   * output gate:                   head h of row t is multiplied by sigmoid(out_gate[t][h])        (out_gate = nullptr: off)
 // Scores, soft-max weights and the output accumulation are fp32 whatever the cache holds.
 //
 // One launch serves every row of a forward, prefill portions and decoded tokens alike: row t belongs to sequence row_seq[t] at
@@ -92,10 +96,26 @@ __device__ __forceinline__ float ga_dot(const T* __restrict__ k, const float* __
     return acc;
 }
 
-constexpr int kGaMaxDim = 256;  // key / value size limit of the row kernel (q in LDS, four value channels per lane)
+constexpr int kGaMaxDim = 1024;  // key size limit of the row kernel (q in LDS); value size: 64 * VC, VC value channels per lane
+
+__device__ __forceinline__ int ga_first_key(const GeneralAttnParams& p, int pos)
+{
+    return p.chunk > 0 ? pos / p.chunk * p.chunk : 0;
+}
+
+// where head h of an output row starts: heads side by side unless the caller spaces them (a batched product reads them at a stride)
+__device__ __forceinline__ size_t ga_out_head(const GeneralAttnParams& p, int h)
+{
+    return (size_t)h * (p.out_head_stride > 0 ? p.out_head_stride : p.vdim);
+}
+
+__device__ __forceinline__ float ga_out_gate(const GeneralAttnParams& p, int t, int h)
+{
+    return p.out_gate ? 1.f / (1.f + expf(-p.out_gate[(size_t)t * p.ld_gate + h])) : 1.f;
+}
 
 // grid (rows, ceil(q_heads / 4), splits), 256 threads: wave w -> head blockIdx.y * 4 + w
-template<class T>
+template<class T, int VC>
 __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
 {
     __shared__ float qs[4][kGaMaxDim];
@@ -114,9 +134,15 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
     }
     const float qscale = p.scale * ga_query_temp(p, pos);
     const int   nkeys = pos + 1, nblk = (nkeys + p.block_len - 1) / p.block_len;
-    const int   per = (nblk + p.splits - 1) / p.splits;
-    const int   b0 = sp * per, b1 = min(nblk, b0 + per);
-    float m = -1e30f, l = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+    const int   first = ga_first_key(p, pos), bf = first / p.block_len;  // the first visible key and its block
+    const int   per = (nblk - bf + p.splits - 1) / p.splits;
+    const int   b0 = bf + sp * per, b1 = min(nblk, b0 + per);
+    const float r1 = p.dist_r1 ? p.dist_r1[h] : 0.f, r2 = p.dist_r1 ? p.dist_r2[h] : 0.f;
+    float m = -1e30f, l = 0.f, o[VC];
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+        o[c] = 0.f;
+    }
     // LDS writes of this wave are read by this wave only: a wave barrier is enough
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -126,12 +152,16 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
         const T*    kb   = (const T*)base + (size_t)g * p.block_len * D;
         const T*    vb   = (const T*)(base + p.v_offset) + (size_t)g * p.block_len * V;  // [V][block_len]
         const int   n    = min(p.block_len, nkeys - b * p.block_len);
-        for (int j0 = 0; j0 < n; j0 += 64) {
+        const int   jlo  = first - b * p.block_len;  // keys below it lie in an earlier chunk
+        for (int j0 = max(0, jlo) / 64 * 64; j0 < n; j0 += 64) {
             const int  j     = j0 + lane;
-            const bool valid = j < n;
+            const bool valid = j < n && j >= jlo;
             float      sc    = -1e30f;
             if (valid) {
                 sc = ga_modify(p, ga_dot<T>(kb + (size_t)j * D, qs[wave], D), qscale);
+                if (p.dist_r1) {
+                    sc -= r1 * log1pf(r2 * (float)(pos - (b * p.block_len + j)));
+                }
             }
             const float m_new = fmaxf(m, ga_wave_max(sc));
             const float alpha = __expf(m - m_new);
@@ -139,15 +169,15 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
             l                 = l * alpha + ga_wave_sum(pj);
             m                 = m_new;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
+            for (int c = 0; c < VC; ++c) {
                 o[c] *= alpha;
             }
             const int cnt = min(64, n - j0);
-            for (int jj = 0; jj < cnt; ++jj) {
+            for (int jj = max(0, jlo - j0); jj < cnt; ++jj) {
                 const float w  = __shfl(pj, jj);
                 const T*    vr = vb + (j0 + jj);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
+                for (int c = 0; c < VC; ++c) {
                     const int v = lane + 64 * c;
                     if (v < V) {
                         o[c] = fmaf(w, (float)vr[(size_t)v * p.block_len], o[c]);
@@ -165,9 +195,10 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
         else {
             inv = 1.f / l;
         }
-        T* out = (T*)p.out + (size_t)t * p.ldo + (size_t)h * V;
+        inv *= ga_out_gate(p, t, h);
+        T* out = (T*)p.out + (size_t)t * p.ldo + ga_out_head(p, h);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < VC; ++c) {
             const int v = lane + 64 * c;
             if (v < V) {
                 out[v] = (T)(o[c] * inv);
@@ -178,7 +209,7 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
     float* po = p.partial_o + (((size_t)t * p.q_heads + h) * p.splits + sp) * V;
     float* pm = p.partial_ml + (((size_t)t * p.q_heads + h) * p.splits + sp) * 2;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < VC; ++c) {
         const int v = lane + 64 * c;
         if (v < V) {
             po[v] = o[c];
@@ -191,7 +222,7 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
 }
 
 // merge of the key splits (+ the sink): grid (rows, q_heads), 64 threads
-template<class T>
+template<class T, int VC>
 __global__ __launch_bounds__(64) void attn_rows_merge_kernel(GeneralAttnParams p)
 {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, V = p.vdim;
@@ -202,25 +233,52 @@ __global__ __launch_bounds__(64) void attn_rows_merge_kernel(GeneralAttnParams p
         mf = fmaxf(mf, pm[s * 2]);
     }
     float l = p.sink ? __expf(p.sink[h] - mf) : 0.f;
-    float o[4] = {0.f, 0.f, 0.f, 0.f};
+    float o[VC];
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+        o[c] = 0.f;
+    }
     for (int s = 0; s < p.splits; ++s) {
         const float a = __expf(pm[s * 2] - mf);
         l += a * pm[s * 2 + 1];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < VC; ++c) {
             const int v = lane + 64 * c;
             if (v < V) {
                 o[c] = fmaf(a, po[(size_t)s * V + v], o[c]);
             }
         }
     }
-    T* out = (T*)p.out + (size_t)t * p.ldo + (size_t)h * V;
+    const float inv = ga_out_gate(p, t, h) / l;
+    T* out = (T*)p.out + (size_t)t * p.ldo + ga_out_head(p, h);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < VC; ++c) {
         const int v = lane + 64 * c;
         if (v < V) {
-            out[v] = (T)(o[c] / l);
+            out[v] = (T)(o[c] * inv);
         }
+    }
+}
+
+template<class T>
+static void launch_rows_merge(const GeneralAttnParams& p, hipStream_t st)
+{
+    if (p.vdim <= 256) {
+        attn_rows_merge_kernel<T, 4><<<dim3(p.rows, p.q_heads), 64, 0, st>>>(p);
+    }
+    else {
+        attn_rows_merge_kernel<T, 16><<<dim3(p.rows, p.q_heads), 64, 0, st>>>(p);
+    }
+}
+
+template<class T>
+static void launch_rows(const GeneralAttnParams& p, dim3 grid, hipStream_t st)
+{
+    if (p.vdim <= 256) {
+        attn_rows_kernel<T, 4><<<grid, 256, 0, st>>>(p);
+    }
+    else {
+        attn_rows_kernel<T, 16><<<grid, 256, 0, st>>>(p);
     }
 }
 
@@ -232,7 +290,8 @@ size_t general_attention_workspace_bytes(int rows, int q_heads, int vdim, int sp
 int launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st)
 {
     TM_REQUIRE(p.rows >= 0 && p.q_heads >= 1 && p.kv_heads >= 1 && p.q_heads % p.kv_heads == 0, "attention: head counts");
-    TM_REQUIRE(p.dim >= 1 && p.dim <= kGaMaxDim && p.vdim >= 1 && p.vdim <= kGaMaxDim, "attention: 1 <= dim, vdim <= 256");
+    TM_REQUIRE(p.dim >= 1 && p.dim <= kGaMaxDim && p.vdim >= 1 && p.vdim <= kGaMaxDim, "attention: 1 <= dim, vdim <= 1024");
+    TM_REQUIRE(p.chunk >= 0 && (!p.dist_r1 || p.dist_r2) && (!p.out_gate || p.ld_gate >= p.q_heads), "attention: chunk / distance penalty / gate");
     TM_REQUIRE(p.block_len >= 1 && p.splits >= 1 && (p.splits == 1 || (p.partial_o && p.partial_ml)), "attention: splits / workspace");
     TM_REQUIRE(p.elem_bytes == 2 || p.elem_bytes == 4, "attention: bf16 or fp32");
     TM_REQUIRE(p.qtemp_coef == 0.f || p.qtemp_every > 0.f, "attention: query temperature period");
@@ -241,18 +300,18 @@ int launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st)
     }
     const dim3 grid(p.rows, (p.q_heads + 3) / 4, p.splits);
     if (p.elem_bytes == 2) {
-        attn_rows_kernel<__bf16><<<grid, 256, 0, st>>>(p);
+        launch_rows<__bf16>(p, grid, st);
     }
     else {
-        attn_rows_kernel<float><<<grid, 256, 0, st>>>(p);
+        launch_rows<float>(p, grid, st);
     }
     TM_HIP_CHECK(hipGetLastError());
     if (p.splits > 1) {
         if (p.elem_bytes == 2) {
-            attn_rows_merge_kernel<__bf16><<<dim3(p.rows, p.q_heads), 64, 0, st>>>(p);
+            launch_rows_merge<__bf16>(p, st);
         }
         else {
-            attn_rows_merge_kernel<float><<<dim3(p.rows, p.q_heads), 64, 0, st>>>(p);
+            launch_rows_merge<float>(p, st);
         }
         TM_HIP_CHECK(hipGetLastError());
     }
@@ -280,10 +339,13 @@ __device__ __forceinline__ float ga_tanh_fast(float x)
 // Every key / value fragment is loaded ONCE and serves all RT row tiles; the value fragments are requested before the soft-max
 // arithmetic so that their latency hides under it.  qf: the rows' query fragments; limit: last visible key of the lane's rows
 // (block-relative; < 0: none); kb / vb: the key head's keys [64][D] and transposed values [V][64] of this block.
+// lower: first visible key of the lane's rows (block-relative, may be negative); r1 / r2: the distance penalty of the lane's rows' head
+// (r1 * log2(1 + r2 * (limit - key)) leaves the score, which lives in the log2 domain; bias = false: none)
 template<int DS, int VT, int RT, bool MASK, bool EAGER>
 __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const __bf16* __restrict__ kb, const __bf16* __restrict__ vb, int D,
-                                              int V, const int (&limit)[RT], const float (&qscale)[RT], float cap, float inv_cap,
-                                              float (&m)[RT], float (&l)[RT], floatx4 (&o)[RT][VT])
+                                              int V, const int (&limit)[RT], const int (&lower)[RT], const float (&qscale)[RT], float cap,
+                                              float inv_cap, bool bias, float r1, float r2, float (&m)[RT], float (&l)[RT],
+                                              floatx4 (&o)[RT][VT])
 {
     const int    lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -348,9 +410,12 @@ __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const 
                 if (cap > 0.f) {
                     v = fmaf(__builtin_amdgcn_rcpf(fast_exp2(v) + 1.f), -2.f * cap2, cap2);
                 }
+                const int key = (kt >> 1) * 32 + lg * 8 + (kt & 1) * 4 + r;
+                if (bias) {  // (a key ahead of the row gives the logarithm of a number that may be negative: the mask below discards it)
+                    v = fmaf(-r1, __builtin_amdgcn_logf(fmaf(r2, (float)(limit[rt] - key), 1.f)), v);
+                }
                 if (MASK) {
-                    const int key = (kt >> 1) * 32 + lg * 8 + (kt & 1) * 4 + r;
-                    v             = key <= limit[rt] ? v : -1e30f;
+                    v = (key <= limit[rt] && key >= lower[rt]) ? v : -1e30f;
                 }
                 sc[rt][kt][r] = v;
                 bmax          = fmaxf(bmax, v);
@@ -360,12 +425,13 @@ __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const 
         bmax = fmaxf(bmax, __shfl_xor(bmax, 32));
         const float m_new = fmaxf(m[rt], bmax);
         const float alpha = fast_exp2(m[rt] - m_new);
+        const float m_ref = fmaxf(m_new, -1e29f);  // a row that has seen no key yet (its chunk starts behind this block): every weight is 0
         float       bsum  = 0.f;
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float e = fast_exp2(sc[rt][kt][r] - m_new);  // a masked score is -1e30: 2^(-1e30 - m) = 0 (a row sees its own key: m is finite)
+                const float e = fast_exp2(sc[rt][kt][r] - m_ref);  // a masked score is -1e30: 2^(-1e30 - m) = 0
                 bsum += e;
                 pf[rt][kt >> 1][(kt & 1) * 4 + r] = (__bf16)e;
             }
@@ -412,7 +478,9 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
     const float cap = p.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
     bf16x8  qf[RT][DS];  // B operand of S^T: row = lane % 16, channels ds * 32 + (lane / 16) * 8 .. + 8
     float   qscale[RT], m[RT], l[RT];
-    int     pos[RT];
+    int     pos[RT], first[RT];
+    const bool  bias = p.dist_r1 != nullptr;
+    const float r1 = bias ? p.dist_r1[h] : 0.f, r2 = bias ? p.dist_r2[h] : 0.f;
     bool    q_ok[RT];
     floatx4 o[RT][VT];
 #pragma unroll
@@ -420,6 +488,7 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
         const int qi = row0 + rt * 16 + lr;
         q_ok[rt]     = qi < q_len;
         pos[rt]      = pos0 + qi;
+        first[rt]    = ga_first_key(p, pos[rt]);
         const __bf16* q = (const __bf16*)p.q + (size_t)(row_base + (q_ok[rt] ? qi : 0)) * p.ldq + (size_t)h * D;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
@@ -437,19 +506,22 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
     }
     const int last_pos = pos0 + min(q_len, row0 + 16 * RT) - 1;  // the wave's last row sees keys 0 .. last_pos
     const int nblk     = last_pos / 64 + 1;
-    for (int b = 0; b < nblk; ++b) {
+    const int first_lo = ga_first_key(p, pos0 + row0), first_hi = ga_first_key(p, last_pos);  // of the wave's first and last row
+    for (int b = first_lo / 64; b < nblk; ++b) {
         const char* base = (const char*)table[b] + p.layer_offset;
-        int         limit[RT];
+        int         limit[RT], lower[RT];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             limit[rt] = q_ok[rt] ? pos[rt] - b * 64 : -1;
+            lower[rt] = first[rt] - b * 64;
         }
         const __bf16 *kb = (const __bf16*)base + (size_t)g * 64 * D, *vb = (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V;
-        if (b * 64 + 63 <= pos0 + row0) {  // every row of the wave sees the whole block (rows beyond the portion are discarded anyway)
-            ga_block_step<DS, VT, RT, false, false>(qf, kb, vb, D, V, limit, qscale, cap, inv_cap, m, l, o);
+        // every row of the wave sees the whole block (rows beyond the portion are discarded anyway)
+        if (b * 64 + 63 <= pos0 + row0 && b * 64 >= first_hi) {
+            ga_block_step<DS, VT, RT, false, false>(qf, kb, vb, D, V, limit, lower, qscale, cap, inv_cap, bias, r1, r2, m, l, o);
         }
         else {
-            ga_block_step<DS, VT, RT, true, false>(qf, kb, vb, D, V, limit, qscale, cap, inv_cap, m, l, o);
+            ga_block_step<DS, VT, RT, true, false>(qf, kb, vb, D, V, limit, lower, qscale, cap, inv_cap, bias, r1, r2, m, l, o);
         }
     }
 #pragma unroll
@@ -465,8 +537,9 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
         else {
             inv = 1.f / l[rt];
         }
+        inv *= ga_out_gate(p, row_base + row0 + rt * 16 + lr, h);
         // lane holds O[row lr][channel t * 16 + lg * 4 + r]
-        __bf16* out = (__bf16*)p.out + (size_t)(row_base + row0 + rt * 16 + lr) * p.ldo + (size_t)h * V;
+        __bf16* out = (__bf16*)p.out + (size_t)(row_base + row0 + rt * 16 + lr) * p.ldo + ga_out_head(p, h);
 #pragma unroll
         for (int t = 0; t < VT; ++t) {
 #pragma unroll
@@ -515,13 +588,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, i
     for (int v = 0; v < VT; ++v) {
         o1[0][v] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    const int nblk = pos / 64 + 1, per = (nblk + p.splits - 1) / p.splits;
-    const int b0 = sp * per, b1 = min(nblk, b0 + per);
+    const bool  bias = p.dist_r1 != nullptr;
+    const float r1 = bias ? p.dist_r1[h] : 0.f, r2 = bias ? p.dist_r2[h] : 0.f;  // of the lane's head
+    const int first = ga_first_key(p, pos), bf = first / 64;
+    const int nblk = pos / 64 + 1, per = (nblk - bf + p.splits - 1) / p.splits;
+    const int b0 = bf + sp * per, b1 = min(nblk, b0 + per);
     for (int b = b0 + wave; b < b1; b += 4) {
         const char* base = (const char*)table[b] + p.layer_offset;
-        const int limit[1] = {pos - b * 64};
+        const int limit[1] = {pos - b * 64}, lower[1] = {first - b * 64};
         ga_block_step<DS, VT, 1, true, true>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D,
-                                       V, limit, qscale, cap, inv_cap, m1, l1, o1);
+                                       V, limit, lower, qscale, cap, inv_cap, bias, r1, r2, m1, l1, o1);
     }
     const float m = m1[0] * kLn2, l = l1[0];  // back from the log2 domain: the merge below and the split merge kernel use e^x
     floatx4 (&o)[VT] = o1[0];
@@ -568,7 +644,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, i
         else {
             inv = 1.f / lt;
         }
-        __bf16* out = (__bf16*)p.out + (size_t)t * p.ldo + (size_t)h * V;
+        inv *= ga_out_gate(p, t, h);
+        __bf16* out = (__bf16*)p.out + (size_t)t * p.ldo + ga_out_head(p, h);
 #pragma unroll
         for (int v = 0; v < VT; ++v) {
 #pragma unroll
@@ -663,7 +740,7 @@ int launch_general_attention_decode(const GeneralAttnParams& p, hipStream_t st)
     const int chunks = (p.q_heads / p.kv_heads + 15) / 16;
     TM_TRY_RC(launch_mfma(p, chunks, dim3(p.rows, p.kv_heads * chunks, p.splits), st, true));
     if (p.splits > 1) {
-        attn_rows_merge_kernel<__bf16><<<dim3(p.rows, p.q_heads), 64, 0, st>>>(p);
+        launch_rows_merge<__bf16>(p, st);
         TM_HIP_CHECK(hipGetLastError());
     }
     return 0;

@@ -77,19 +77,36 @@ struct LmLayer {
     float *       norm1 = nullptr, *norm2 = nullptr, *sink = nullptr;
     int           n_q = 0, n_k = 0, n_v = 0, n_att = 0;  // heads * dim, kv_heads * dim, kv_heads * vdim, heads * vdim
     int64_t       kv_offset = 0, v_offset = 0;           // this layer's keys inside a cache block; its values behind the keys
+    // blocks whose projections leave the fused product in fp32 (per-head norms, rotation, gates and routers read them): `qkv` then holds
+    // every projection of the block's input h side by side, columns
+    //   attention: [q | k | v | out gate | residual gate 1 | residual gate 2 | router]     latent: [q | dkv | residual gate 1 | 2 | router]
+    bool          wide = false;
+    int           a_dim = 0, a_vdim = 0, a_kv = 0;       // what the attention kernel sees (latent: kv_rank + rot_dim, kv_rank, 1)
+    int           c_k = 0, c_v = 0, c_g = 0, c_rg1 = 0, c_rg2 = 0, c_router = 0;  // columns of the fused projection
+    int           plain_stride = 0, lat_stride = 0;      // latent: head strides of the unrotated query parts / of the latent attention output
+    DenseWeight   wo, gu, down;      // output projection; [gate | up] along N; down (experts: one image per expert in gu / down)
+    DenseWeight   uk, uv;            // latent: key expansion transposed [kv_rank][dim] and value expansion [vdim][kv_rank], one image per head
+    float *       r1 = nullptr, *r2 = nullptr, *rg1_b = nullptr, *rg2_b = nullptr, *c_norm = nullptr, *inv_freq = nullptr;
 };
 
 struct LayeredModel {
     tm_layered_config    cfg{};
     std::vector<LmLayer> layers;
     DenseWeight          head;
+    DenseWeight          loop_in;               // [width][2 width]: the mix of stream and embedding output at the start of a loop pass
+    float*               loop_step = nullptr;   // [loop_times][width]
     void*                embed      = nullptr;  // [vocab][width] bf16 | fp32
     float*               final_norm = nullptr;
     int                  elem       = 2;        // bytes of an activation / cache element
     int                  ldw = 0, ldqkv = 0, ldcat = 0, ldv16 = 0;  // leading dimensions: normed rows, projections, [attention | ff], fp16 logits
+    int                  ldproj = 0, ldq = 0, ldplain = 0, ldlat = 0, ldgu = 0, ldff = 0, ld2w = 0, max_top = 0;
     int                  max_logit_rows = 0;
     float*               d_res = nullptr;       // residual stream [max_tokens][width]
     void *               d_h1 = nullptr, *d_h2 = nullptr, *d_qkv = nullptr, *d_cat = nullptr, *d_hn = nullptr;
+    // wide blocks: fused projection (fp32), queries, unrotated query parts, latent attention output, [gate | up] (fp32), activations
+    float *              d_proj = nullptr, *d_gu = nullptr, *d_x0 = nullptr, *d_moe_y = nullptr, *d_topk_w = nullptr;
+    void *               d_q = nullptr, *d_plain = nullptr, *d_lat = nullptr, *d_ff = nullptr, *d_xx = nullptr, *d_moe_x = nullptr;
+    int *                d_topk_ids = nullptr, *d_offsets = nullptr, *d_f2n = nullptr, *d_en2f = nullptr;
     float*               d_logits_f32 = nullptr;  // [max_logit_rows][vocab]
     int *                d_row_seq = nullptr, *d_row_pos = nullptr, *d_iota = nullptr, *d_want = nullptr, *d_seq_slot = nullptr;
     int *                d_step_ids = nullptr, *d_step_cu_q = nullptr, *d_step_k_len = nullptr;
@@ -98,6 +115,7 @@ struct LayeredModel {
     int                  decode_splits = 1;
     int                  debug_layers  = -1;  // >= 0: the forward stops behind this many layers (parity tests read the residual stream)
     std::map<int64_t, int> sess_len;          // open sessions (scheduler request id) -> tokens held
+    std::map<std::string, int> fan_in;        // tensor name -> input size (synthetic weights: N(0, 1 / fan_in))
 };
 
 // the rows of one forward that share a block table and a (cu_q, k_len) description

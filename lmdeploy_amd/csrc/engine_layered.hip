@@ -9,6 +9,18 @@
 //   cat[:, heads * vdim :] = act(h2 . Wup^T)         activation in the GEMM epilogue
 //   x       += residual_mult * (cat . [Wo | Wdown]^T)   ONE GEMM over the concatenated inputs closes the block in its epilogue
 // The residual stream x is fp32; h, q, k, v, cat and the cache are bf16 (TM_DTYPE_BF16) or fp32 (TM_DTYPE_F32).
+//
+// "Wide" blocks (LmLayer::wide: per-head norms, rotation, gates or routers read the projections in fp32) run
+//   x        = loop.in [x | x0] + loop.step[t]          only where a loop pass begins (concat + GEMM with a bias epilogue)
+//   h        = norm1(x)
+//   proj     = h . [q | k | v | gates | router]^T       ONE GEMM, fp32 output
+//   queries, cache  <- proj                             launch_attn_prep (unit norms) | launch_latent_prep (norm, rotation)
+//   latent:  q[:, head, 0:C] = q_plain[:, head] . uk_head          one batched GEMM (the key expansion carried to the query)
+//   attention (chunk, distance penalty, sink, output gate as parameters)
+//   latent:  cat[:, head] = lat[:, head] . uv_head^T               one batched GEMM (the value expansion)
+//   x       += sigmoid(proj[rg1] + b1) * (cat . Wo^T)              GEMM with the gated-residual epilogue
+//   dense:   gu = h . [gate | up]^T (fp32); a = act(gate) * up; x += sigmoid(proj[rg2] + b2) * (a . Wdown^T)
+//   experts: router top-k -> rows sorted by expert, scaled by their score -> the same two products batched over the experts -> gated sum
 #include "engine_internal.h"
 
 namespace tmk {
@@ -52,6 +64,13 @@ static std::string lname(int i, const char* t)
     return "l" + std::to_string(i) + "." + t;
 }
 
+// blocks whose projections are read in fp32 before they become queries, cache entries, gates or router scores
+static bool layer_wide(const tm_layer_spec& s)
+{
+    return s.mixer == TM_MIXER_LATENT || s.one_norm || s.resid_gate || s.qk_unit_norm || s.v_unit_norm || s.out_gate || s.mlp == TM_MLP_GATED
+           || s.mlp == TM_MLP_MOE;
+}
+
 static int to_f32(tm_engine* e, const std::string& name, size_t n, float** out)
 {
     Slot& s = e->slots[name];
@@ -62,11 +81,85 @@ static int to_f32(tm_engine* e, const std::string& name, size_t n, float** out)
     return 0;
 }
 
-static int place(tm_engine* e, DenseWeight& d, int row0, int col0, const std::string& name, int rows, int cols)
+static int place(tm_engine* e, DenseWeight& d, int row0, int col0, const std::string& name, int rows, int cols, size_t src_row = 0, int item = 0,
+                 bool transpose = false)
 {
     Slot& s = e->slots[name];
     TM_REQUIRE(s.filled, "weight not loaded: " + name);
-    return dense_weight_place(d, row0, col0, s.dev, rows, cols, e->stream);
+    TM_REQUIRE((int64_t)(src_row + rows) * cols * 2 <= s.bytes, "internal: weight part outside " + name);
+    return dense_weight_place(d, row0, col0, (const uint16_t*)s.dev + src_row * cols, rows, cols, e->stream, item, transpose);
+}
+
+static int process_wide_layer(tm_engine* e, int i, LmLayer& L, int dt)
+{
+    const tm_layer_spec& s = L.spec;
+    const int            W = e->lm->cfg.width, H = s.heads;
+    int                  n = L.n_q;
+    TM_TRY(dense_weight_alloc(L.qkv, W, L.c_router + (s.mlp == TM_MLP_MOE ? s.experts : 0), dt, e->stream));
+    TM_TRY(place(e, L.qkv, 0, 0, lname(i, "mix.q"), L.n_q, W));
+    if (s.mixer == TM_MIXER_LATENT) {
+        const int C = s.kv_rank, R = s.rot_dim;
+        TM_TRY(place(e, L.qkv, L.c_k, 0, lname(i, "mix.dkv"), C + R, W));
+        TM_TRY(to_f32(e, lname(i, "mix.dkv.norm"), C, &L.c_norm));
+        TM_TRY(dense_weight_alloc(L.uk, s.dim, C, dt, e->stream, H));
+        TM_TRY(dense_weight_alloc(L.uv, C, s.vdim, dt, e->stream, H));
+        for (int h = 0; h < H; ++h) {  // uk rows [h dim, (h + 1) dim) are head h's [dim][kv_rank]: stored transposed, kv_rank outputs of dim inputs
+            TM_TRY(place(e, L.uk, 0, 0, lname(i, "mix.uk"), s.dim, C, (size_t)h * s.dim, h, true));
+            TM_TRY(place(e, L.uv, 0, 0, lname(i, "mix.uv"), s.vdim, C, (size_t)h * s.vdim, h, false));
+        }
+        std::vector<float> f(R / 2);
+        for (int j = 0; j < R / 2; ++j) {
+            f[j] = (float)std::pow((double)s.rot_base, -2.0 * j / R);
+        }
+        TM_TRY(dmalloc(&L.inv_freq, (size_t)std::max(1, R / 2)));
+        TM_HIP_CHECK(hipMemcpyAsync(L.inv_freq, f.data(), f.size() * 4, hipMemcpyHostToDevice, e->stream));
+        TM_HIP_CHECK(hipStreamSynchronize(e->stream));
+    }
+    else {
+        TM_TRY(place(e, L.qkv, L.c_k, 0, lname(i, "mix.k"), L.a_kv * s.dim, W));
+        TM_TRY(place(e, L.qkv, L.c_v, 0, lname(i, "mix.v"), L.a_kv * s.vdim, W));
+        if (s.out_gate) {
+            TM_TRY(place(e, L.qkv, L.c_g, 0, lname(i, "mix.g"), H, W));
+        }
+    }
+    (void)n;
+    if (s.dist_bias) {
+        TM_TRY(to_f32(e, lname(i, "mix.r1"), H, &L.r1));
+        TM_TRY(to_f32(e, lname(i, "mix.r2"), H, &L.r2));
+    }
+    if (s.sink) {
+        TM_TRY(to_f32(e, lname(i, "mix.sink"), H, &L.sink));
+    }
+    TM_TRY(to_f32(e, lname(i, "norm1"), W, &L.norm1));
+    TM_TRY(dense_weight_alloc(L.wo, L.n_att, W, dt, e->stream));
+    TM_TRY(place(e, L.wo, 0, 0, lname(i, "mix.o"), W, L.n_att));
+    if (s.resid_gate) {
+        TM_TRY(place(e, L.qkv, L.c_rg1, 0, lname(i, "rg1"), W, W));
+        TM_TRY(to_f32(e, lname(i, "rg1.b"), W, &L.rg1_b));
+        if (s.mlp) {
+            TM_TRY(place(e, L.qkv, L.c_rg2, 0, lname(i, "rg2"), W, W));
+            TM_TRY(to_f32(e, lname(i, "rg2.b"), W, &L.rg2_b));
+        }
+    }
+    if (s.mlp == TM_MLP_GATED) {
+        TM_TRY(dense_weight_alloc(L.gu, W, 2 * s.ff, dt, e->stream));
+        TM_TRY(place(e, L.gu, 0, 0, lname(i, "mlp.gate"), s.ff, W));
+        TM_TRY(place(e, L.gu, s.ff, 0, lname(i, "mlp.up"), s.ff, W));
+        TM_TRY(dense_weight_alloc(L.down, s.ff, W, dt, e->stream));
+        TM_TRY(place(e, L.down, 0, 0, lname(i, "mlp.down"), W, s.ff));
+    }
+    else if (s.mlp == TM_MLP_MOE) {
+        TM_TRY(place(e, L.qkv, L.c_router, 0, lname(i, "mlp.router"), s.experts, W));
+        TM_TRY(dense_weight_alloc(L.gu, W, 2 * s.ff, dt, e->stream, s.experts));
+        TM_TRY(dense_weight_alloc(L.down, s.ff, W, dt, e->stream, s.experts));
+        for (int x = 0; x < s.experts; ++x) {
+            const std::string ex = "mlp.e" + std::to_string(x) + ".";
+            TM_TRY(place(e, L.gu, 0, 0, lname(i, (ex + "gate").c_str()), s.ff, W, 0, x));
+            TM_TRY(place(e, L.gu, s.ff, 0, lname(i, (ex + "up").c_str()), s.ff, W, 0, x));
+            TM_TRY(place(e, L.down, 0, 0, lname(i, (ex + "down").c_str()), W, s.ff, 0, x));
+        }
+    }
+    return 0;
 }
 
 int layered_process_weights(tm_engine* e)
@@ -81,6 +174,10 @@ int layered_process_weights(tm_engine* e)
             continue;
         }
         const tm_layer_spec& s = L.spec;
+        if (L.wide) {
+            TM_TRY(process_wide_layer(e, i, L, dt));
+            continue;
+        }
         TM_TRY(dense_weight_alloc(L.qkv, W, L.n_q + L.n_k + L.n_v, dt, e->stream));
         TM_TRY(place(e, L.qkv, 0, 0, lname(i, "mix.q"), L.n_q, W));
         TM_TRY(place(e, L.qkv, L.n_q, 0, lname(i, "mix.k"), L.n_k, W));
@@ -104,7 +201,14 @@ int layered_process_weights(tm_engine* e)
         if (L.src != i) {
             const LmLayer& S = lm.layers[L.src];
             L.qkv = S.qkv, L.up = S.up, L.out = S.out, L.norm1 = S.norm1, L.norm2 = S.norm2, L.sink = S.sink;
+            L.wo = S.wo, L.gu = S.gu, L.down = S.down, L.uk = S.uk, L.uv = S.uv;
+            L.r1 = S.r1, L.r2 = S.r2, L.rg1_b = S.rg1_b, L.rg2_b = S.rg2_b, L.c_norm = S.c_norm, L.inv_freq = S.inv_freq;
         }
+    }
+    if (c.loop_times > 0) {
+        TM_TRY(dense_weight_alloc(lm.loop_in, 2 * W, W, dt, e->stream));
+        TM_TRY(place(e, lm.loop_in, 0, 0, "loop.in", W, 2 * W));
+        TM_TRY(to_f32(e, "loop.step", (size_t)c.loop_times * W, &lm.loop_step));
     }
     TM_TRY(dense_weight_alloc(lm.head, W, c.vocab, dt, e->stream));
     TM_TRY(place(e, lm.head, 0, 0, "head", c.vocab, W));
@@ -145,15 +249,27 @@ int layered_init_synthetic(tm_engine* e, uint64_t seed)
             TM_HIP_CHECK(hipMalloc(&s.dev, s.bytes));
         }
         const size_t cnt  = (size_t)s.bytes / 2;
-        const bool   vec  = n.find("norm") != std::string::npos || n.find("sink") != std::string::npos;
-        // matrices: N(0, 1 / in_features) keeps every projection's output at the scale of its input; vectors: small, around zero
-        float        stdv = 0.02f;
+        const LayeredModel& lm  = *e->lm;
+        const size_t        dot = n.rfind('.');
+        const std::string   leaf = dot == std::string::npos ? n : n.substr(dot + 1);
+        const bool          isnorm = n.find("norm") != std::string::npos;
+        const bool          vec = isnorm || leaf == "sink" || leaf == "r1" || leaf == "r2" || leaf == "b" || leaf == "step";
+        // matrices: N(0, 1 / in_features) keeps every projection's output at the scale of its input; vectors: small, around zero (norm
+        // weights around 1 - norm_offset; distance-penalty numbers positive)
+        float stdv = 0.02f, mean = 0.f;
+        if (isnorm) {
+            mean = 1.f - lm.cfg.norm_offset;
+        }
+        else if (leaf == "r1" || leaf == "r2") {
+            mean = 0.5f;
+        }
         if (!vec && n != "embed") {
-            const LayeredModel& lm = *e->lm;
-            int                 K  = lm.cfg.width;
-            const size_t        dot = n.rfind('.');
-            const std::string   leaf = dot == std::string::npos ? n : n.substr(dot + 1);
-            if (leaf == "o" || leaf == "down") {
+            int  K  = lm.cfg.width;
+            auto fi = lm.fan_in.find(n);
+            if (fi != lm.fan_in.end()) {
+                K = fi->second;
+            }
+            else if (leaf == "o" || leaf == "down") {
                 K = (int)(cnt / lm.cfg.width);
             }
             stdv = 1.0f / std::sqrt((float)K);
@@ -161,7 +277,7 @@ int layered_init_synthetic(tm_engine* e, uint64_t seed)
         else if (n == "embed") {
             stdv = 1.0f;
         }
-        fill_normal_bf16_kernel<<<(cnt + 255) / 256, 256, 0, e->stream>>>((uint16_t*)s.dev, cnt, 0.f, stdv, ++sd);
+        fill_normal_bf16_kernel<<<(cnt + 255) / 256, 256, 0, e->stream>>>((uint16_t*)s.dev, cnt, mean, stdv, ++sd);
         TM_HIP_CHECK(hipGetLastError());
         s.filled = true;
     }
@@ -190,24 +306,69 @@ int layered_start(tm_engine* e)
     e->max_tokens         = std::max(B, std::max(64, c.max_prefill_token_num));
     const size_t T        = e->max_tokens;
     // cache block: every layer run has its keys [kv_heads][block_len][dim] and, behind them, its values transposed [kv_heads][vdim][block_len]
+    lm.ldw      = (m.width + 31) / 32 * 32;
     int64_t off = 0;
-    int     max_qkv = 0, max_cat = 0, max_vdim = 0, max_heads = 0;
+    int     max_qkv = 8, max_cat = 32, max_vdim = 0, max_heads = 0;
+    int     max_proj = 0, max_q = 0, max_plain = 0, max_lat = 0, max_gu = 0, max_ff = 0;
+    bool    any_moe = false;
     for (LmLayer& L : lm.layers) {
         L.kv_offset = off;
         L.v_offset  = (int64_t)L.n_k * c.cache_block_seq_len * lm.elem;
         off += (int64_t)(L.n_k + L.n_v) * c.cache_block_seq_len * lm.elem;
         off         = (off + 15) / 16 * 16;
-        max_qkv     = std::max(max_qkv, L.qkv.N);
-        max_cat     = std::max(max_cat, L.out.Kp);
-        max_vdim    = std::max(max_vdim, L.spec.vdim);
+        max_vdim    = std::max(max_vdim, L.a_vdim);
         max_heads   = std::max(max_heads, L.spec.heads);
+        if (!L.wide) {
+            max_qkv = std::max(max_qkv, L.qkv.N);
+            max_cat = std::max(max_cat, L.out.Kp);
+            continue;
+        }
+        max_cat   = std::max(max_cat, L.wo.Kp);
+        max_proj  = std::max(max_proj, L.qkv.N);
+        max_q     = std::max(max_q, L.spec.heads * L.a_dim);
+        max_plain = std::max(max_plain, L.spec.heads * L.plain_stride);
+        max_lat   = std::max(max_lat, L.spec.heads * L.lat_stride);
+        if (L.spec.mlp) {
+            max_gu     = std::max(max_gu, L.gu.N);
+            max_ff     = std::max(max_ff, L.down.Kp);
+            lm.max_top = std::max(lm.max_top, L.spec.mlp == TM_MLP_MOE ? L.spec.top : 1);
+            any_moe    = any_moe || L.spec.mlp == TM_MLP_MOE;
+        }
     }
     e->block_bytes = off;
-    lm.ldw   = (m.width + 31) / 32 * 32;
     lm.ldqkv = (max_qkv + 31) / 32 * 32;
     lm.ldcat = max_cat;
     lm.ldv16 = e->vocab_local;
     lm.max_logit_rows = (int)std::max<size_t>(B, std::min<size_t>(T, 1024));
+    if (max_proj > 0) {  // wide blocks
+        const size_t TT = T * std::max(1, lm.max_top);  // rows of the experts' products: one per (token, chosen expert)
+        lm.ldproj  = (max_proj + 3) / 4 * 4;
+        lm.ldq     = (max_q + 31) / 32 * 32;
+        lm.ldplain = std::max(32, max_plain);
+        lm.ldlat   = std::max(32, max_lat);
+        lm.ldgu    = std::max(4, (max_gu + 3) / 4 * 4);
+        lm.ldff    = std::max(32, max_ff);
+        TM_TRY(lm_alloc(&lm.d_proj, T * lm.ldproj, st));
+        TM_TRY(lm_alloc((char**)&lm.d_q, T * lm.ldq * lm.elem, st));
+        TM_TRY(lm_alloc((char**)&lm.d_plain, T * lm.ldplain * lm.elem, st));
+        TM_TRY(lm_alloc((char**)&lm.d_lat, T * lm.ldlat * lm.elem, st));
+        TM_TRY(lm_alloc(&lm.d_gu, TT * lm.ldgu, st));
+        TM_TRY(lm_alloc((char**)&lm.d_ff, TT * lm.ldff * lm.elem, st));
+        if (any_moe) {
+            TM_TRY(lm_alloc((char**)&lm.d_moe_x, TT * lm.ldw * lm.elem, st));
+            TM_TRY(lm_alloc(&lm.d_moe_y, TT * m.width, st));
+            TM_TRY(lm_alloc(&lm.d_topk_w, TT, st));
+            TM_TRY(lm_alloc(&lm.d_topk_ids, TT, st));
+            TM_TRY(lm_alloc(&lm.d_f2n, TT, st));
+            TM_TRY(lm_alloc(&lm.d_en2f, TT, st));
+            TM_TRY(lm_alloc(&lm.d_offsets, (size_t)1026, st));
+        }
+    }
+    if (m.loop_times > 0) {
+        lm.ld2w = lm.loop_in.Kp;
+        TM_TRY(lm_alloc(&lm.d_x0, T * m.width, st));
+        TM_TRY(lm_alloc((char**)&lm.d_xx, T * lm.ld2w * lm.elem, st));
+    }
     TM_TRY(lm_alloc(&lm.d_res, T * m.width, st));
     TM_TRY(lm_alloc((char**)&lm.d_h1, T * lm.ldw * lm.elem, st));
     TM_TRY(lm_alloc((char**)&lm.d_h2, T * lm.ldw * lm.elem, st));
@@ -284,7 +445,8 @@ void layered_free(tm_engine* e)
         LmLayer& L = lm.layers[i];
         if (L.src == (int)i) {
             dense_weight_free(L.qkv), dense_weight_free(L.up), dense_weight_free(L.out);
-            for (float* p : {L.norm1, L.norm2, L.sink}) {
+            dense_weight_free(L.wo), dense_weight_free(L.gu), dense_weight_free(L.down), dense_weight_free(L.uk), dense_weight_free(L.uv);
+            for (float* p : {L.norm1, L.norm2, L.sink, L.r1, L.r2, L.rg1_b, L.rg2_b, L.c_norm, L.inv_freq}) {
                 if (p) {
                     (void)hipFree(p);
                 }
@@ -292,6 +454,13 @@ void layered_free(tm_engine* e)
         }
     }
     dense_weight_free(lm.head);
+    dense_weight_free(lm.loop_in);
+    for (void* p : {(void*)lm.loop_step, (void*)lm.d_proj, (void*)lm.d_gu, (void*)lm.d_x0, (void*)lm.d_moe_y, (void*)lm.d_topk_w, lm.d_q, lm.d_plain, lm.d_lat,
+                    lm.d_ff, lm.d_xx, lm.d_moe_x, (void*)lm.d_topk_ids, (void*)lm.d_offsets, (void*)lm.d_f2n, (void*)lm.d_en2f}) {
+        if (p) {
+            (void)hipFree(p);
+        }
+    }
     for (void* p : {(void*)lm.embed, (void*)lm.final_norm, (void*)lm.d_res, lm.d_h1, lm.d_h2, lm.d_qkv, lm.d_cat, lm.d_hn, (void*)lm.d_logits_f32,
                     (void*)lm.d_row_seq, (void*)lm.d_row_pos, (void*)lm.d_iota, (void*)lm.d_want, (void*)lm.d_seq_slot, (void*)lm.d_step_ids,
                     (void*)lm.d_step_cu_q, (void*)lm.d_step_k_len, (void*)lm.d_attn_ws}) {
@@ -310,6 +479,22 @@ static GeneralAttnParams attn_params(tm_engine* e, const LmLayer& L, const LmPar
     p.out          = (char*)lm.d_cat + (size_t)P.row0 * lm.ldcat * lm.elem;
     p.ldq          = lm.ldqkv;
     p.ldo          = lm.ldcat;
+    if (L.wide) {
+        p.q   = (const char*)lm.d_q + (size_t)P.row0 * lm.ldq * lm.elem;
+        p.ldq = lm.ldq;
+        if (L.spec.mixer == TM_MIXER_LATENT) {  // the attention output stays in the latent space until the value expansion
+            p.out             = (char*)lm.d_lat + (size_t)P.row0 * lm.ldlat * lm.elem;
+            p.ldo             = lm.ldlat;
+            p.out_head_stride = L.lat_stride;
+        }
+        if (L.spec.out_gate) {
+            p.out_gate = lm.d_proj + (size_t)P.row0 * lm.ldproj + L.c_g;
+            p.ld_gate  = lm.ldproj;
+        }
+    }
+    p.dist_r1 = L.r1;
+    p.dist_r2 = L.r2;
+    p.chunk   = L.spec.chunk;
     p.rows         = P.rows;
     p.row_seq      = lm.d_row_seq + P.row0;
     p.row_pos      = lm.d_row_pos + P.row0;
@@ -321,9 +506,9 @@ static GeneralAttnParams attn_params(tm_engine* e, const LmLayer& L, const LmPar
     p.block_len    = e->cfg.cache_block_seq_len;
     p.elem_bytes   = lm.elem;
     p.q_heads      = L.spec.heads;
-    p.kv_heads     = L.spec.kv_heads;
-    p.dim          = L.spec.dim;
-    p.vdim         = L.spec.vdim;
+    p.kv_heads     = L.a_kv;
+    p.dim          = L.a_dim;
+    p.vdim         = L.a_vdim;
     p.scale        = L.spec.scale;
     p.softcap      = L.spec.softcap;
     p.qtemp_coef   = L.spec.qtemp_coef;
@@ -334,6 +519,92 @@ static GeneralAttnParams attn_params(tm_engine* e, const LmLayer& L, const LmPar
     p.cu_q         = P.cu_q;
     p.k_len        = P.k_len;
     return p;
+}
+
+// one wide block over M rows (see the head of this file)
+static int wide_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts, int nparts)
+{
+    LayeredModel&            lm = *e->lm;
+    const tm_layered_config& m  = lm.cfg;
+    const tm_layer_spec&     s  = L.spec;
+    hipStream_t              st = e->stream;
+    const int                W = m.width, H = s.heads;
+    const bool               latent = s.mixer == TM_MIXER_LATENT;
+    TM_PROF(P_RES_NORM, TM_TRY(launch_rmsnorm_f32(lm.d_h1, nullptr, lm.ldw, lm.elem, lm.d_res, nullptr, L.norm1, nullptr, m.norm_offset, m.norm_eps,
+                                                  M, W, st)));
+    TM_PROF(P_GEMM_QKV, TM_TRY(launch_dense_linear(L.qkv, lm.d_h1, lm.ldw, lm.d_proj, lm.ldproj, M, kDenseScaleF32, 1.f, st)));
+    for (int i = 0; i < nparts; ++i) {
+        const LmPart&     P    = parts[i];
+        GeneralAttnParams p    = attn_params(e, L, P);
+        const float*      proj = lm.d_proj + (size_t)P.row0 * lm.ldproj;
+        if (latent) {
+            TM_PROF(P_KV_STORE, TM_TRY(launch_latent_prep(proj, lm.ldproj, 0, L.c_k, (char*)lm.d_plain + (size_t)P.row0 * lm.ldplain * lm.elem, lm.ldplain,
+                                                          L.plain_stride, (void*)p.q, lm.ldq, L.c_norm, L.inv_freq, s.dim, s.rot_dim, s.kv_rank,
+                                                          m.norm_eps, p, st)));
+        }
+        else {
+            TM_PROF(P_KV_STORE, TM_TRY(launch_attn_prep(proj, lm.ldproj, 0, L.c_k, L.c_v, (void*)p.q, lm.ldq, s.qk_unit_norm != 0, s.v_unit_norm != 0,
+                                                        m.norm_eps, p, st)));
+        }
+    }
+    if (latent) {
+        DenseCall c;
+        c.count        = H;
+        c.x_col_stride = L.plain_stride;
+        c.y_col_stride = L.a_dim;
+        TM_PROF(P_GEMM_QKV, TM_TRY(launch_dense_call(L.uk, lm.d_plain, lm.ldplain, lm.d_q, lm.ldq, M, c, st)));
+    }
+    for (int i = 0; i < nparts; ++i) {
+        const LmPart&     P = parts[i];
+        GeneralAttnParams p = attn_params(e, L, P);
+        if (P.decode && lm.decode_splits > 1 && general_attention_workspace_bytes(P.rows, H, L.a_vdim, lm.decode_splits) <= lm.attn_ws_bytes) {
+            p.splits     = lm.decode_splits;
+            p.partial_o  = lm.d_attn_ws;
+            p.partial_ml = lm.d_attn_ws + (size_t)P.rows * H * p.splits * L.a_vdim;
+        }
+        TM_PROF(P_ATTN, TM_TRY(launch_general_attention(p, !P.decode, st)));
+    }
+    if (latent) {
+        DenseCall c;
+        c.count        = H;
+        c.x_col_stride = L.lat_stride;
+        c.y_col_stride = s.vdim;
+        TM_PROF(P_GEMM_O, TM_TRY(launch_dense_call(L.uv, lm.d_lat, lm.ldlat, lm.d_cat, lm.ldcat, M, c, st)));
+    }
+    DenseCall close;  // the sublayer's result joins the stream: gated element by element, or scaled
+    close.epi   = s.resid_gate ? kDenseResidGate : kDenseResidAdd;
+    close.alpha = m.residual_mult;
+    close.ldg   = lm.ldproj;
+    if (s.resid_gate) {
+        close.gate      = lm.d_proj + L.c_rg1;
+        close.gate_bias = L.rg1_b;
+    }
+    TM_PROF(P_GEMM_O, TM_TRY(launch_dense_call(L.wo, lm.d_cat, lm.ldcat, lm.d_res, W, M, close, st)));
+    if (s.resid_gate) {
+        close.gate      = lm.d_proj + L.c_rg2;
+        close.gate_bias = L.rg2_b;
+    }
+    if (s.mlp == TM_MLP_GATED) {
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_linear(L.gu, lm.d_h1, lm.ldw, lm.d_gu, lm.ldgu, M, kDenseScaleF32, 1.f, st)));
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_act_mul(lm.d_ff, lm.ldff, lm.elem, lm.d_gu, lm.ldgu, s.ff, M, s.ff, s.act, st)));
+        TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_call(L.down, lm.d_ff, lm.ldff, lm.d_res, W, M, close, st)));
+    }
+    else if (s.mlp == TM_MLP_MOE) {
+        const int k = s.top, E = s.experts;
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_topk_sigmoid(lm.d_topk_ids, lm.d_topk_w, lm.d_proj + L.c_router, lm.ldproj, M, E, k, st)));
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_route(lm.d_offsets, lm.d_f2n, lm.d_en2f, lm.d_topk_ids, M, E, k, st)));
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_gather(lm.d_moe_x, lm.ldw, lm.d_h1, lm.ldw, lm.elem, lm.d_topk_w, lm.d_en2f, M, W, k, true, st)));
+        DenseCall c;
+        c.epi         = kDenseScaleF32;
+        c.count       = E;
+        c.row_offsets = lm.d_offsets;
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_call(L.gu, lm.d_moe_x, lm.ldw, lm.d_gu, lm.ldgu, M * k, c, st)));
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_act_mul(lm.d_ff, lm.ldff, lm.elem, lm.d_gu, lm.ldgu, s.ff, M * k, s.ff, s.act, st)));
+        TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_call(L.down, lm.d_ff, lm.ldff, lm.d_moe_y, W, M * k, c, st)));
+        TM_PROF(P_GEMM_DOWN, TM_TRY(launch_moe_combine_f32(lm.d_res, lm.d_moe_y, lm.d_topk_w, lm.d_en2f, s.resid_gate ? close.gate : nullptr, lm.ldproj,
+                                                     close.gate_bias, M, W, k, false, st)));
+    }
+    return 0;
 }
 
 // the layer loop over M rows described by `parts`; leaves the residual stream in lm.d_res
@@ -348,10 +619,24 @@ static int layered_layers(tm_engine* e, const int* d_ids, int M, const LmPart* p
         TM_TRY(launch_rows_prepare(lm.d_row_seq + P.row0, lm.d_row_pos + P.row0, P.cu_q, P.k_len, P.nseq, P.rows, st));
     }
     TM_PROF(P_EMBED, TM_TRY(launch_embedding_f32(lm.d_res, lm.embed, lm.elem, d_ids, M, m.width, m.vocab, st)));
+    if (m.loop_times > 0) {  // the embedding output is read again where a loop pass begins
+        TM_PROF(P_EMBED, TM_TRY(launch_embedding_f32(lm.d_x0, lm.embed, lm.elem, d_ids, M, m.width, m.vocab, st)));
+    }
     const int n_run = lm.debug_layers >= 0 ? std::min(lm.debug_layers, m.n_layers) : m.n_layers;
     for (int li = 0; li < n_run; ++li) {
         const LmLayer&       L = lm.layers[li];
         const tm_layer_spec& s = L.spec;
+        if (s.loop_pass >= 0) {
+            DenseCall c;
+            c.epi  = kDenseBiasF32;
+            c.bias = lm.loop_step + (size_t)s.loop_pass * m.width;
+            TM_PROF(P_RES_NORM, TM_TRY(launch_concat2(lm.d_xx, lm.ld2w, lm.elem, lm.d_res, lm.d_x0, M, m.width, st)));
+            TM_PROF(P_GEMM_O, TM_TRY(launch_dense_call(lm.loop_in, lm.d_xx, lm.ld2w, lm.d_res, m.width, M, c, st)));
+        }
+        if (L.wide) {
+            TM_TRY(wide_layer(e, L, M, parts, nparts));
+            continue;
+        }
         TM_PROF(P_RES_NORM, TM_TRY(launch_rmsnorm_f32(lm.d_h1, s.mlp ? lm.d_h2 : nullptr, lm.ldw, lm.elem, lm.d_res, nullptr, L.norm1, L.norm2,
                                                       m.norm_offset, m.norm_eps, M, m.width, st)));
         TM_PROF(P_GEMM_QKV, TM_TRY(launch_dense_linear(L.qkv, lm.d_h1, lm.ldw, lm.d_qkv, lm.ldqkv, M, kDenseStore, 1.f, st)));
@@ -440,10 +725,25 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
     TM_REQUIRE(m->norm_eps > 0.f, "norm_eps > 0");
     for (int i = 0; i < m->n_layers; ++i) {
         const tm_layer_spec& s = m->layers[i];
-        TM_REQUIRE(s.mixer == TM_MIXER_ATTENTION, "layer " + std::to_string(i) + ": unknown mixer");
-        TM_REQUIRE(s.heads >= 1 && s.kv_heads >= 1 && s.heads % s.kv_heads == 0, "layer " + std::to_string(i) + ": heads % kv_heads");
-        TM_REQUIRE(s.dim >= 1 && s.dim <= 256 && s.vdim >= 1 && s.vdim <= 256, "layer " + std::to_string(i) + ": 1 <= dim, vdim <= 256");
-        TM_REQUIRE(s.mlp == TM_MLP_NONE || (s.mlp == TM_MLP_DENSE && s.ff >= 1 && s.act == TM_ACT_RELU2), "layer " + std::to_string(i) + ": feed-forward");
+        const std::string at = "layer " + std::to_string(i);
+        TM_REQUIRE(s.mixer == TM_MIXER_ATTENTION || s.mixer == TM_MIXER_LATENT, at + ": unknown mixer");
+        TM_REQUIRE(s.heads >= 1 && s.kv_heads >= 1 && s.heads % s.kv_heads == 0, at + ": heads % kv_heads");
+        TM_REQUIRE(s.dim >= 1 && s.dim <= 256 && s.vdim >= 1 && s.vdim <= 256, at + ": 1 <= dim, vdim <= 256");
+        TM_REQUIRE(s.chunk >= 0 && s.loop_pass < m->loop_times, at + ": chunk >= 0, loop_pass < loop_times");
+        if (layer_wide(s)) {
+            TM_REQUIRE(s.one_norm, at + ": gates, per-head norms, latent attention and gated feed-forwards read ONE norm of the stream (one_norm)");
+            TM_REQUIRE(s.mlp == TM_MLP_NONE || ((s.mlp == TM_MLP_GATED || s.mlp == TM_MLP_MOE) && s.ff >= 1 && s.act >= TM_ACT_RELU2 && s.act <= TM_ACT_SILU),
+                       at + ": feed-forward");
+            TM_REQUIRE(s.mlp != TM_MLP_MOE || (s.experts >= 1 && s.experts <= 1024 && s.top >= 1 && s.top <= s.experts), at + ": 1 <= top <= experts <= 1024");
+            if (s.mixer == TM_MIXER_LATENT) {
+                TM_REQUIRE(s.kv_heads == 1 && s.kv_rank >= 1 && s.rot_dim >= 0 && s.rot_dim % 2 == 0 && s.kv_rank + s.rot_dim <= 1024 && s.rot_base > 0.f,
+                           at + ": latent attention: kv_heads 1, kv_rank >= 1, rot_dim even, kv_rank + rot_dim <= 1024");
+                TM_REQUIRE(!s.qk_unit_norm && !s.v_unit_norm && !s.out_gate, at + ": latent attention has no per-head unit norms and no output gate");
+            }
+        }
+        else {
+            TM_REQUIRE(s.mlp == TM_MLP_NONE || (s.mlp == TM_MLP_DENSE && s.ff >= 1 && s.act == TM_ACT_RELU2), at + ": feed-forward");
+        }
         TM_REQUIRE(s.qtemp_coef == 0.f || s.qtemp_every > 0.f, "layer " + std::to_string(i) + ": query temperature period");
         TM_REQUIRE(s.weights_of < 0 || (s.weights_of < m->n_layers && s.weights_of != i && m->layers[s.weights_of].weights_of < 0),
                    "layer " + std::to_string(i) + ": weights_of must name a layer with tensors of its own");
@@ -452,6 +752,9 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
             TM_REQUIRE(o.heads == s.heads && o.kv_heads == s.kv_heads && o.dim == s.dim && o.vdim == s.vdim && o.mlp == s.mlp && o.ff == s.ff
                            && o.sink == s.sink,
                        "layer " + std::to_string(i) + ": sizes differ from the layer whose weights it uses");
+            TM_REQUIRE(layer_wide(o) == layer_wide(s) && o.mixer == s.mixer && o.kv_rank == s.kv_rank && o.rot_dim == s.rot_dim && o.experts == s.experts
+                           && o.resid_gate == s.resid_gate && o.out_gate == s.out_gate && o.dist_bias == s.dist_bias,
+                       "layer " + std::to_string(i) + ": form differs from the layer whose weights it uses");
         }
     }
     TM_HIP_CHECK(hipSetDevice(c->device));
@@ -481,6 +784,80 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
         L.n_k      = L.spec.kv_heads * L.spec.dim;
         L.n_v      = L.spec.kv_heads * L.spec.vdim;
         L.n_att    = L.spec.heads * L.spec.vdim;
+        L.a_dim = L.spec.dim, L.a_vdim = L.spec.vdim, L.a_kv = L.spec.kv_heads;
+        L.wide = layer_wide(L.spec);
+        auto slot = [&](const std::string& name, int64_t rows, int64_t cols) {
+            e->slots[name].bytes = rows * cols * 2;
+            lm.fan_in[name]      = (int)cols;
+        };
+        if (L.wide) {
+            const tm_layer_spec& s = L.spec;
+            const int            H = s.heads;
+            int                  next;
+            if (s.mixer == TM_MIXER_LATENT) {  // the cache holds one key head [kv_rank | rot_dim] and the latent vector as its value
+                L.a_dim = s.kv_rank + s.rot_dim, L.a_vdim = s.kv_rank, L.a_kv = 1;
+                L.n_q = H * (s.dim + s.rot_dim), L.n_k = L.a_dim, L.n_v = L.a_vdim;
+                L.plain_stride = (s.dim + 31) / 32 * 32, L.lat_stride = (s.kv_rank + 31) / 32 * 32;
+                L.c_k = L.n_q;
+                next  = L.c_k + s.kv_rank + s.rot_dim;
+            }
+            else {
+                L.c_k = L.n_q, L.c_v = L.c_k + L.n_k, L.c_g = L.c_v + L.n_v;
+                next  = L.c_g + (s.out_gate ? H : 0);
+            }
+            L.c_rg1 = next, next += s.resid_gate ? (int)W : 0;
+            L.c_rg2 = next, next += s.resid_gate && s.mlp ? (int)W : 0;
+            L.c_router = next;
+            if (L.src != i) {
+                continue;
+            }
+            slot(lname(i, "norm1"), 1, W);
+            slot(lname(i, "mix.q"), L.n_q, W);
+            slot(lname(i, "mix.o"), W, L.n_att);
+            if (s.mixer == TM_MIXER_LATENT) {
+                slot(lname(i, "mix.dkv"), s.kv_rank + s.rot_dim, W);
+                slot(lname(i, "mix.dkv.norm"), 1, s.kv_rank);
+                slot(lname(i, "mix.uk"), (int64_t)H * s.dim, s.kv_rank);
+                slot(lname(i, "mix.uv"), (int64_t)H * s.vdim, s.kv_rank);
+            }
+            else {
+                slot(lname(i, "mix.k"), L.n_k, W);
+                slot(lname(i, "mix.v"), L.n_v, W);
+                if (s.out_gate) {
+                    slot(lname(i, "mix.g"), H, W);
+                }
+            }
+            if (s.dist_bias) {
+                slot(lname(i, "mix.r1"), 1, H);
+                slot(lname(i, "mix.r2"), 1, H);
+            }
+            if (s.sink) {
+                slot(lname(i, "mix.sink"), 1, H);
+            }
+            if (s.resid_gate) {
+                slot(lname(i, "rg1"), W, W);
+                slot(lname(i, "rg1.b"), 1, W);
+                if (s.mlp) {
+                    slot(lname(i, "rg2"), W, W);
+                    slot(lname(i, "rg2.b"), 1, W);
+                }
+            }
+            if (s.mlp == TM_MLP_GATED) {
+                slot(lname(i, "mlp.gate"), s.ff, W);
+                slot(lname(i, "mlp.up"), s.ff, W);
+                slot(lname(i, "mlp.down"), W, s.ff);
+            }
+            else if (s.mlp == TM_MLP_MOE) {
+                slot(lname(i, "mlp.router"), s.experts, W);
+                for (int x = 0; x < s.experts; ++x) {
+                    const std::string ex = "mlp.e" + std::to_string(x) + ".";
+                    slot(lname(i, (ex + "gate").c_str()), s.ff, W);
+                    slot(lname(i, (ex + "up").c_str()), s.ff, W);
+                    slot(lname(i, (ex + "down").c_str()), W, s.ff);
+                }
+            }
+            continue;
+        }
         if (L.src != i) {
             continue;
         }
@@ -497,6 +874,11 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
             e->slots[lname(i, "mlp.up")].bytes   = W * L.spec.ff * 2;
             e->slots[lname(i, "mlp.down")].bytes = W * L.spec.ff * 2;
         }
+    }
+    if (m->loop_times > 0) {
+        e->slots["loop.in"].bytes   = W * 2 * W * 2;
+        lm.fan_in["loop.in"]        = (int)(2 * W);
+        e->slots["loop.step"].bytes = (int64_t)m->loop_times * W * 2;
     }
     e->slots["embed"].bytes      = W * m->vocab * 2;
     e->slots["final.norm"].bytes = W * 2;

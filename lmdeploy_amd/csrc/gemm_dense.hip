@@ -14,7 +14,12 @@
 //
 // The epilogue is chosen per call (DenseEpilogue): plain store, relu(x)^2 (the squared-ReLU feed-forward), accumulate into the fp32
 // residual stream with a multiplier (resid += alpha * acc: the output projection of a residual block closes the block in the GEMM),
-// or alpha * acc as fp32 (scaled logits).
+// or alpha * acc as fp32 (scaled logits), acc + bias[n] as fp32, or the sigmoid-gated residual sum
+// resid += sigmoid(gate[m][n] + gate_bias[n]) * acc (a block whose sublayers are gated element by element).
+//
+// A launch may be BATCHED (DenseCall::count > 1, grid z): item g multiplies with image g of the weight (images at a fixed stride), reads
+// x at column g * x_col_stride and writes y at column g * y_col_stride -- per-head projections of one activation row -- or, with
+// row_offsets, owns the rows [row_offsets[g], row_offsets[g + 1]) of x and y: the experts of a mixture over rows sorted by expert.
 #include "tm_kernels.h"
 
 namespace tmk {
@@ -22,22 +27,45 @@ namespace tmk {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 template<class T>
-__device__ __forceinline__ void dense_epilogue(void* y, int ldy, int m, int n, float acc, int epi, float alpha)
+__device__ __forceinline__ void dense_epilogue(void* y, int ldy, int m, int n, float acc, const DenseCall& c)
 {
     const size_t i = (size_t)m * ldy + n;
-    if (epi == kDenseStore) {
+    if (c.epi == kDenseStore) {
         ((T*)y)[i] = (T)acc;
     }
-    else if (epi == kDenseRelu2) {
+    else if (c.epi == kDenseRelu2) {
         const float r = fmaxf(acc, 0.f);
         ((T*)y)[i]    = (T)(r * r);
     }
-    else if (epi == kDenseResidAdd) {
-        ((float*)y)[i] += alpha * acc;
+    else if (c.epi == kDenseResidAdd) {
+        ((float*)y)[i] += c.alpha * acc;
     }
-    else {
-        ((float*)y)[i] = alpha * acc;
+    else if (c.epi == kDenseScaleF32) {
+        ((float*)y)[i] = c.alpha * acc;
     }
+    else if (c.epi == kDenseBiasF32) {
+        ((float*)y)[i] = acc + c.bias[n];
+    }
+    else {  // kDenseResidGate
+        const float z = c.gate[(size_t)m * c.ldg + n] + c.gate_bias[n];
+        ((float*)y)[i] += acc / (1.f + expf(-z));
+    }
+}
+
+// the item of a batched launch: where its operands start, and its row count (<= 0: nothing to do)
+struct DenseItem {
+    size_t x_off, w_off;
+    int    row_base, col_base, M;
+};
+__device__ __forceinline__ DenseItem dense_item(const DenseCall& c, int g, int M, int ldx)
+{
+    DenseItem it{(size_t)g * c.x_col_stride, (size_t)g * c.w_stride, 0, g * c.y_col_stride, M};
+    if (c.row_offsets) {
+        it.row_base = c.row_offsets[g];
+        it.x_off += (size_t)it.row_base * ldx;
+        it.M = c.row_offsets[g + 1] - it.row_base;
+    }
+    return it;
 }
 
 // ---- bf16, M <= 32 ------------------------------------------------------------------------------------------------------------
@@ -50,9 +78,15 @@ __device__ __forceinline__ void dense_epilogue(void* y, int ldy, int m, int n, f
 
 template<int MT, int NT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void dense_skinny_bf16_kernel(const __bf16* __restrict__ x, int ldx, const __bf16* __restrict__ w, int Kp,
-                                                                void* __restrict__ y, int ldy, int M, int N, int epi, float alpha)
+                                                                void* __restrict__ y, int ldy, int M, int N, DenseCall call)
 {
     __shared__ float red[WAVES][MT * NT][64][4];
+    const DenseItem it = dense_item(call, blockIdx.y, M, ldx);
+    const int       row_base = it.row_base, col_base = it.col_base;
+    M = it.M, x += it.x_off, w += it.w_off;
+    if (M <= 0) {
+        return;
+    }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0   = blockIdx.x * 16 * NT;
     const int r    = lane & 15, kc = (lane >> 4) * 8;
@@ -153,7 +187,7 @@ __global__ __launch_bounds__(WAVES * 64) void dense_skinny_bf16_kernel(const __b
         // C fragment: column = lane % 16, rows (lane / 16) * 4 + i
         const int m = (tj / NT) * 16 + (l >> 4) * 4 + i, n = n0 + (tj % NT) * 16 + (l & 15);
         if (m < M && n < N) {
-            dense_epilogue<__bf16>(y, ldy, m, n, s, epi, alpha);
+            dense_epilogue<__bf16>(y, ldy, row_base + m, col_base + n, s, call);
         }
     }
 }
@@ -162,12 +196,18 @@ __global__ __launch_bounds__(WAVES * 64) void dense_skinny_bf16_kernel(const __b
 constexpr int kTM = 128, kTN = 128, kTK = 32, kLdsRow = kTK + 8;  // 80-byte LDS rows: 16-byte fragment reads of 16 rows hit all banks once
 
 __global__ __launch_bounds__(256) void dense_tiled_bf16_kernel(const __bf16* __restrict__ x, int ldx, const __bf16* __restrict__ w, int Kp,
-                                                               void* __restrict__ y, int ldy, int M, int N, int epi, float alpha)
+                                                               void* __restrict__ y, int ldy, int M, int N, DenseCall call)
 {
     __shared__ __attribute__((aligned(16))) __bf16 sa[2][kTM * kLdsRow];
     __shared__ __attribute__((aligned(16))) __bf16 sb[2][kTN * kLdsRow];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m0 = blockIdx.y * kTM, n0 = blockIdx.x * kTN;
+    const DenseItem it = dense_item(call, blockIdx.z, M, ldx);
+    const int       row_base = it.row_base, col_base = it.col_base;
+    M = it.M, x += it.x_off, w += it.w_off;
+    if (m0 >= M) {  // the whole workgroup: an item with fewer rows than the launch's largest
+        return;
+    }
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
     // staging: 128 rows x 32 k = 512 16-byte vectors per operand, two per thread: vector v -> row v / 4, k chunk (v % 4) * 8
     const int  sr0 = tid >> 2, sr1 = sr0 + 64, sk = (tid & 3) * 8;
@@ -238,7 +278,7 @@ __global__ __launch_bounds__(256) void dense_tiled_bf16_kernel(const __bf16* __r
             for (int q = 0; q < 4; ++q) {
                 const int m = m0 + wm + i * 16 + (lane >> 4) * 4 + q, n = n0 + wn + j * 16 + (lane & 15);
                 if (m < M && n < N) {
-                    dense_epilogue<__bf16>(y, ldy, m, n, acc[i][j][q], epi, alpha);
+                    dense_epilogue<__bf16>(y, ldy, row_base + m, col_base + n, acc[i][j][q], call);
                 }
             }
         }
@@ -249,12 +289,18 @@ __global__ __launch_bounds__(256) void dense_tiled_bf16_kernel(const __bf16* __r
 // 64 x 64 x 16 tiles, 256 threads, 4 x 4 outputs per thread; operands transposed into LDS ([k][row]) so that a thread's four rows /
 // columns are one 16-byte read.  fmaf in k order: the result of a row does not depend on what shares its tile.
 __global__ __launch_bounds__(256) void dense_f32_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w, int Kp,
-                                                        void* __restrict__ y, int ldy, int M, int N, int epi, float alpha)
+                                                        void* __restrict__ y, int ldy, int M, int N, DenseCall call)
 {
     __shared__ __attribute__((aligned(16))) float sa[16][64 + 4];
     __shared__ __attribute__((aligned(16))) float sb[16][64 + 4];
     const int tid = threadIdx.x;
     const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    const DenseItem it = dense_item(call, blockIdx.z, M, ldx);
+    const int       row_base = it.row_base, col_base = it.col_base;
+    M = it.M, x += it.x_off, w += it.w_off;
+    if (m0 >= M) {
+        return;
+    }
     const int tr = (tid >> 4) * 4, tc = (tid & 15) * 4;
     const int lr = tid >> 2, lk = (tid & 3) * 4;  // staging: row lr (0..63), k chunk lk (0, 4, 8, 12)
     const bool   ain = m0 + lr < M;
@@ -290,7 +336,7 @@ __global__ __launch_bounds__(256) void dense_f32_kernel(const float* __restrict_
         for (int j = 0; j < 4; ++j) {
             const int m = m0 + tr + i, n = n0 + tc + j;
             if (m < M && n < N) {
-                dense_epilogue<float>(y, ldy, m, n, acc[i][j], epi, alpha);
+                dense_epilogue<float>(y, ldy, row_base + m, col_base + n, acc[i][j], call);
             }
         }
     }
@@ -307,43 +353,50 @@ __host__ __device__ inline size_t dense_frag_index(int n, int k, int Kp)
 }
 
 template<class T>
-__global__ void dense_place_kernel(T* __restrict__ dst, int Kp, int row0, int col0, const __bf16* __restrict__ src, int rows, int cols)
+__global__ void dense_place_kernel(T* __restrict__ dst, int Kp, int row0, int col0, const __bf16* __restrict__ src, int rows, int cols,
+                                   int transpose)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < (size_t)rows * cols) {
         const int r = (int)(i / cols), c = (int)(i % cols);
+        const int n = row0 + (transpose ? c : r), k = col0 + (transpose ? r : c);  // transposed: the block's columns become output rows
         if constexpr (sizeof(T) == 2) {
-            dst[dense_frag_index(row0 + r, col0 + c, Kp)] = (T)(float)src[i];
+            dst[dense_frag_index(n, k, Kp)] = (T)(float)src[i];
         }
         else {
-            dst[(size_t)(row0 + r) * Kp + col0 + c] = (T)(float)src[i];
+            dst[(size_t)n * Kp + k] = (T)(float)src[i];
         }
     }
 }
 
-int dense_weight_alloc(DenseWeight& d, int K, int N, int dtype, hipStream_t st)
+int dense_weight_alloc(DenseWeight& d, int K, int N, int dtype, hipStream_t st, int count)
 {
-    TM_REQUIRE(K >= 1 && N >= 1 && (dtype == kDenseBf16 || dtype == kDenseF32), "dense weight: K, N >= 1, dtype bf16 | f32");
+    TM_REQUIRE(K >= 1 && N >= 1 && count >= 1 && (dtype == kDenseBf16 || dtype == kDenseF32), "dense weight: K, N, count >= 1, dtype bf16 | f32");
     d.K     = K;
     d.N     = N;
     d.Kp    = (K + 31) / 32 * 32;
     d.Np    = (N + 127) / 128 * 128;
     d.dtype = dtype;
-    d.bytes = (size_t)d.Kp * d.Np * (dtype == kDenseF32 ? 4 : 2);
+    d.count = count;
+    d.bytes = (size_t)d.Kp * d.Np * count * (dtype == kDenseF32 ? 4 : 2);
     TM_HIP_CHECK(hipMalloc(&d.w, d.bytes));
     TM_HIP_CHECK(hipMemsetAsync(d.w, 0, d.bytes, st));
     return 0;
 }
 
-int dense_weight_place(DenseWeight& d, int row0, int col0, const void* src_bf16, int rows, int cols, hipStream_t st)
+int dense_weight_place(DenseWeight& d, int row0, int col0, const void* src_bf16, int rows, int cols, hipStream_t st, int item, bool transpose)
 {
-    TM_REQUIRE(d.w && row0 >= 0 && col0 >= 0 && row0 + rows <= d.N && col0 + cols <= d.K, "dense weight: part outside the image");
-    const size_t n = (size_t)rows * cols;
+    TM_REQUIRE(d.w && row0 >= 0 && col0 >= 0 && item >= 0 && item < d.count, "dense weight: part outside the image");
+    TM_REQUIRE(row0 + (transpose ? cols : rows) <= d.N && col0 + (transpose ? rows : cols) <= d.K, "dense weight: part outside the image");
+    const size_t n = (size_t)rows * cols, at = (size_t)item * d.Np * d.Kp;
+    if (n == 0) {
+        return 0;
+    }
     if (d.dtype == kDenseF32) {
-        dense_place_kernel<float><<<(n + 255) / 256, 256, 0, st>>>((float*)d.w, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols);
+        dense_place_kernel<float><<<(n + 255) / 256, 256, 0, st>>>((float*)d.w + at, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols, transpose);
     }
     else {
-        dense_place_kernel<__bf16><<<(n + 255) / 256, 256, 0, st>>>((__bf16*)d.w, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols);
+        dense_place_kernel<__bf16><<<(n + 255) / 256, 256, 0, st>>>((__bf16*)d.w + at, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols, transpose);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;
@@ -359,28 +412,43 @@ void dense_weight_free(DenseWeight& d)
 
 int launch_dense_linear(const DenseWeight& d, const void* x, int ldx, void* y, int ldy, int M, int epi, float alpha, hipStream_t st)
 {
-    TM_REQUIRE(d.w && x && y && M >= 0 && ldx >= d.Kp && ldy >= d.N, "dense linear: operands");
-    TM_REQUIRE(epi >= kDenseStore && epi <= kDenseScaleF32, "dense linear: epilogue");
+    DenseCall c;
+    c.epi   = epi;
+    c.alpha = alpha;
+    return launch_dense_call(d, x, ldx, y, ldy, M, c, st);
+}
+
+int launch_dense_call(const DenseWeight& d, const void* x, int ldx, void* y, int ldy, int M, DenseCall call, hipStream_t st)
+{
+    const int epi = call.epi;
+    TM_REQUIRE(d.w && x && y && M >= 0 && call.count >= 1 && call.count <= d.count, "dense linear: operands");
+    TM_REQUIRE(ldx >= d.Kp + (call.count - 1) * call.x_col_stride && ldy >= d.N + (call.count - 1) * call.y_col_stride, "dense linear: row lengths");
+    TM_REQUIRE(epi >= kDenseStore && epi <= kDenseResidGate, "dense linear: epilogue");
+    TM_REQUIRE(epi != kDenseBiasF32 || call.bias, "dense linear: bias");
+    TM_REQUIRE(epi != kDenseResidGate || (call.gate && call.gate_bias && call.ldg >= d.N), "dense linear: gate");
     if (M == 0) {
         return 0;
     }
+    call.w_stride = (size_t)d.Np * d.Kp;
+    const int G   = call.count;
     if (d.dtype == kDenseF32) {
         TM_REQUIRE(ldx % 4 == 0, "dense linear (fp32): rows must be 16-byte aligned");
-        dense_f32_kernel<<<dim3(d.Np / 64, (M + 63) / 64), 256, 0, st>>>((const float*)x, ldx, (const float*)d.w, d.Kp, y, ldy, M, d.N, epi, alpha);
+        TM_REQUIRE(call.x_col_stride % 4 == 0, "dense linear (fp32): items must be 16-byte aligned");
+        dense_f32_kernel<<<dim3(d.Np / 64, (M + 63) / 64, G), 256, 0, st>>>((const float*)x, ldx, (const float*)d.w, d.Kp, y, ldy, M, d.N, call);
     }
     else {
-        TM_REQUIRE(ldx % 8 == 0, "dense linear (bf16): rows must be 16-byte aligned");
+        TM_REQUIRE(ldx % 8 == 0 && call.x_col_stride % 8 == 0, "dense linear (bf16): rows and items must be 16-byte aligned");
         if (M <= 32) {
             // two column tiles per wave where that still leaves >= 512 workgroups (two per CU): wide outputs amortise the activation reads
             const int nt     = d.N >= 512 * 32 ? 2 : 1;
             const int wgs    = (d.N + 16 * nt - 1) / (16 * nt);
             const int chunk  = (nt == 1 ? 8 : 4) * 32;
             int       waves  = 4;  // ... and more waves per workgroup while the device holds fewer than 16 per CU and K has a chunk for each
-            while (waves < (nt == 1 ? 16 : 8) && wgs * waves < 256 * 16 && d.Kp >= chunk * 2 * waves) {
+            while (waves < (nt == 1 ? 16 : 8) && wgs * G * waves < 256 * 16 && d.Kp >= chunk * 2 * waves) {
                 waves *= 2;
             }
 #define TM_SKINNY(MT_, NT_, W_)                                                                                                     \
-    dense_skinny_bf16_kernel<MT_, NT_, W_><<<wgs, W_ * 64, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy, M, d.N, epi, alpha)
+    dense_skinny_bf16_kernel<MT_, NT_, W_><<<dim3(wgs, G), W_ * 64, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy, M, d.N, call)
 #define TM_SKINNY_W(MT_, NT_)                     \
     if (waves == 16 && NT_ == 1) {                \
         TM_SKINNY(MT_, 1, 16);                    \
@@ -411,8 +479,8 @@ int launch_dense_linear(const DenseWeight& d, const void* x, int ldx, void* y, i
 #undef TM_SKINNY
         }
         else {
-            dense_tiled_bf16_kernel<<<dim3(d.Np / kTN, (M + kTM - 1) / kTM), 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y, ldy,
-                                                                                       M, d.N, epi, alpha);
+            dense_tiled_bf16_kernel<<<dim3(d.Np / kTN, (M + kTM - 1) / kTM, G), 256, 0, st>>>((const __bf16*)x, ldx, (const __bf16*)d.w, d.Kp, y,
+                                                                                          ldy, M, d.N, call);
         }
     }
     TM_HIP_CHECK(hipGetLastError());

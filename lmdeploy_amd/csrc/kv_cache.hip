@@ -392,4 +392,147 @@ int launch_kv_store_general(const void* qkv, int ld, int k_col, int v_col, const
     return 0;
 }
 
+// ---- projections of a mixer -> queries + paged cache, from the fp32 output of the fused projection GEMM ------------------------------
+// Grouped-query attention whose queries, keys and values may each be scaled to unit root mean square per head (no weight): one wave per
+// (row, head vector).  proj [rows][ld]: queries at q_col ([q_heads][dim]), keys at k_col ([kv_heads][dim]), values at v_col
+// ([kv_heads][vdim]).  Queries go to q_out [rows][ldq] (head h at h * dim), keys / values into the cache in the general layout.
+template<class T>
+__global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict__ proj, int ld, int q_col, int k_col, int v_col, T* __restrict__ q_out,
+                                                        int ldq, int qk_norm, int v_norm, float eps, GeneralAttnParams p)
+{
+    const int lane = threadIdx.x & 63, t = blockIdx.x, u = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int H = p.q_heads, G = p.kv_heads;
+    if (u >= H + 2 * G) {
+        return;
+    }
+    const int    kind = u < H ? 0 : (u < H + G ? 1 : 2), head = kind == 0 ? u : (kind == 1 ? u - H : u - H - G);
+    const int    n    = kind == 2 ? p.vdim : p.dim;
+    const float* x    = proj + (size_t)t * ld + (kind == 0 ? q_col : (kind == 1 ? k_col : v_col)) + (size_t)head * n;
+    float        inv  = 1.f;
+    if (kind == 2 ? v_norm : qk_norm) {
+        float ss = 0.f;
+        for (int i = lane; i < n; i += 64) {
+            ss = fmaf(x[i], x[i], ss);
+        }
+        inv = 1.0f / sqrtf(group_sum<64>(ss) / (float)n + eps);
+    }
+    if (kind == 0) {
+        T* q = q_out + (size_t)t * ldq + (size_t)head * n;
+        for (int i = lane; i < n; i += 64) {
+            q[i] = (T)(x[i] * inv);
+        }
+        return;
+    }
+    const int s = p.row_seq[t], pos = p.row_pos[t], ti = pos % p.block_len;
+    char* base = (char*)p.block_ptrs[(size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride + pos / p.block_len] + p.layer_offset;
+    if (kind == 1) {
+        T* k = (T*)base + ((size_t)head * p.block_len + ti) * n;
+        for (int i = lane; i < n; i += 64) {
+            k[i] = (T)(x[i] * inv);
+        }
+    }
+    else {
+        T* v = (T*)(base + p.v_offset) + (size_t)head * n * p.block_len + ti;
+        for (int i = lane; i < n; i += 64) {
+            v[(size_t)i * p.block_len] = (T)(x[i] * inv);
+        }
+    }
+}
+
+int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col, void* q_out, int ldq, bool qk_norm, bool v_norm, float eps,
+                     const GeneralAttnParams& p, hipStream_t st)
+{
+    TM_REQUIRE(proj && q_out && p.row_seq && p.row_pos && p.block_ptrs && p.block_stride >= 1, "attn_prep: operands");
+    if (p.rows == 0) {
+        return 0;
+    }
+    const dim3 grid(p.rows, (p.q_heads + 2 * p.kv_heads + 3) / 4);
+    if (p.elem_bytes == 2) {
+        attn_prep_kernel<__bf16><<<grid, 256, 0, st>>>(proj, ld, q_col, k_col, v_col, (__bf16*)q_out, ldq, qk_norm, v_norm, eps, p);
+    }
+    else {
+        attn_prep_kernel<float><<<grid, 256, 0, st>>>(proj, ld, q_col, k_col, v_col, (float*)q_out, ldq, qk_norm, v_norm, eps, p);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+// Latent attention: per token ONE normed latent vector c (size C) and ONE rotated key part (size R) shared by all heads are cached; a
+// head's keys and values are linear images of c.  The cache entry is the key [c | rotated part] (p.dim = C + R, one key head) and the
+// value c (p.vdim = C): attention then runs in the latent space -- the query's unrotated part is carried through the key expansion
+// beforehand (q_plain . (U c) = (U^T q_plain) . c), the value expansion is applied to the attention output.
+// proj [rows][ld]: queries at q_col, head h as [D unrotated | R rotated]; at dkv_col the C latent channels, then the R rotated ones.
+//   q_plain [rows][ldp], head h at h * plain_stride : unrotated query parts (input of the key-expansion product)
+//   q_full  [rows][ldq], head h at h * (C + R)      : the rotated part goes to [C, C + R) (the product fills [0, C))
+// Rotation pairs channel i with i + R / 2; angle = position * inv_freq[i], fp32.
+template<class T>
+__global__ __launch_bounds__(256) void latent_prep_kernel(const float* __restrict__ proj, int ld, int q_col, int dkv_col, T* __restrict__ q_plain,
+                                                          int ldp, int plain_stride, T* __restrict__ q_full, int ldq,
+                                                          const float* __restrict__ c_norm_w, const float* __restrict__ inv_freq, int D, int R, int C,
+                                                          float eps, GeneralAttnParams p)
+{
+    __shared__ float red[4];
+    const int    t = blockIdx.x, H = p.q_heads, half = R / 2;
+    const int    s = p.row_seq[t], pos = p.row_pos[t], ti = pos % p.block_len;
+    const float* x = proj + (size_t)t * ld;
+    for (int i = threadIdx.x; i < H * D; i += 256) {
+        const int h = i / D, d = i % D;
+        q_plain[(size_t)t * ldp + (size_t)h * plain_stride + d] = (T)x[q_col + h * (D + R) + d];
+    }
+    for (int i = threadIdx.x; i < H * half; i += 256) {
+        const int   h = i / half, f = i % half;
+        const float u = x[q_col + h * (D + R) + D + f], v = x[q_col + h * (D + R) + D + f + half];
+        float       sn, cs;
+        sincosf((float)pos * inv_freq[f], &sn, &cs);
+        T* q = q_full + (size_t)t * ldq + (size_t)h * (C + R) + C;
+        q[f]        = (T)(u * cs - v * sn);
+        q[f + half] = (T)(v * cs + u * sn);
+    }
+    char* base = (char*)p.block_ptrs[(size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride + pos / p.block_len] + p.layer_offset;
+    T*    k    = (T*)base + (size_t)ti * (C + R);
+    T*    vt   = (T*)(base + p.v_offset) + ti;
+    float ss   = 0.f;
+    for (int i = threadIdx.x; i < C; i += 256) {
+        ss = fmaf(x[dkv_col + i], x[dkv_col + i], ss);
+    }
+    ss = group_sum<64>(ss);
+    if ((threadIdx.x & 63) == 0) {
+        red[threadIdx.x >> 6] = ss;
+    }
+    __syncthreads();
+    const float inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)C + eps);
+    for (int i = threadIdx.x; i < C; i += 256) {
+        const T c = (T)(x[dkv_col + i] * inv * c_norm_w[i]);
+        k[i]                          = c;
+        vt[(size_t)i * p.block_len] = c;
+    }
+    for (int f = threadIdx.x; f < half; f += 256) {
+        const float u = x[dkv_col + C + f], v = x[dkv_col + C + f + half];
+        float       sn, cs;
+        sincosf((float)pos * inv_freq[f], &sn, &cs);
+        k[C + f]        = (T)(u * cs - v * sn);
+        k[C + f + half] = (T)(v * cs + u * sn);
+    }
+}
+
+int launch_latent_prep(const float* proj, int ld, int q_col, int dkv_col, void* q_plain, int ldp, int plain_stride, void* q_full, int ldq,
+                       const float* c_norm_w, const float* inv_freq, int D, int R, int C, float eps, const GeneralAttnParams& p, hipStream_t st)
+{
+    TM_REQUIRE(proj && q_plain && q_full && c_norm_w && inv_freq && p.row_seq && p.row_pos && p.block_ptrs, "latent_prep: operands");
+    TM_REQUIRE(R % 2 == 0 && p.kv_heads == 1 && p.dim == C + R && p.vdim == C && plain_stride >= D, "latent_prep: sizes");
+    if (p.rows == 0) {
+        return 0;
+    }
+    if (p.elem_bytes == 2) {
+        latent_prep_kernel<__bf16><<<p.rows, 256, 0, st>>>(proj, ld, q_col, dkv_col, (__bf16*)q_plain, ldp, plain_stride, (__bf16*)q_full, ldq, c_norm_w,
+                                                           inv_freq, D, R, C, eps, p);
+    }
+    else {
+        latent_prep_kernel<float><<<p.rows, 256, 0, st>>>(proj, ld, q_col, dkv_col, (float*)q_plain, ldp, plain_stride, (float*)q_full, ldq, c_norm_w,
+                                                          inv_freq, D, R, C, eps, p);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
 }  // namespace tmk

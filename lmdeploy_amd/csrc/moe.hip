@@ -340,4 +340,105 @@ void moe_free(MoeBlock& m)
     m.groups13_p8 = m.groups2_p8 = nullptr;
 }
 
+// ---- mixture of experts on the fp32 residual stream (layer-list family) -------------------------------------------------------------
+// Router scores sigmoid(logit) from fp32 logits; the `k` largest win (ties: the lower index); the weights are the scores as they are.
+__global__ void moe_topk_sigmoid_kernel(int* __restrict__ ids, float* __restrict__ w, const float* __restrict__ logits, int ld, int T, int E, int k)
+{
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= T) {
+        return;
+    }
+    const float* z = logits + (size_t)t * ld;
+    for (int j = 0; j < k; ++j) {
+        int   best = -1;
+        float bz   = 0.f;
+        for (int e = 0; e < E; ++e) {
+            bool taken = false;
+            for (int q = 0; q < j; ++q) {
+                taken = taken || ids[(size_t)t * k + q] == e;
+            }
+            if (!taken && (best < 0 || z[e] > bz)) {  // the sigmoid is monotonic: order by the logit
+                best = e;
+                bz   = z[e];
+            }
+        }
+        ids[(size_t)t * k + j] = best;
+        w[(size_t)t * k + j]   = 1.f / (1.f + expf(-bz));
+    }
+}
+
+int launch_moe_topk_sigmoid(int* ids, float* w, const float* logits, int ld, int T, int E, int k, hipStream_t st)
+{
+    TM_REQUIRE(ids && w && logits && E >= 1 && k >= 1 && k <= E && ld >= E, "moe top-k: operands");
+    if (T == 0) {
+        return 0;
+    }
+    moe_topk_sigmoid_kernel<<<(T + 63) / 64, 64, 0, st>>>(ids, w, logits, ld, T, E, k);
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+// rows sorted by expert: xs[en2f[j][t]] = (scale ? w[t][j] : 1) * x[t] -- the weight on the expert's INPUT
+template<class T>
+__global__ __launch_bounds__(256) void moe_gather_kernel(T* __restrict__ xs, int lds, const T* __restrict__ x, int ldx, const float* __restrict__ w,
+                                                         const int* __restrict__ en2f, int Tn, int H, int k, int scale)
+{
+    const int t = blockIdx.x / k, j = blockIdx.x % k;
+    const int f = en2f[(size_t)j * Tn + t];
+    const float a = scale ? w[(size_t)t * k + j] : 1.f;
+    for (int i = threadIdx.x; i < H; i += 256) {
+        xs[(size_t)f * lds + i] = (T)(a * (float)x[(size_t)t * ldx + i]);
+    }
+}
+
+int launch_moe_gather(void* xs, int lds, const void* x, int ldx, int elem_bytes, const float* w, const int* en2f, int T, int H, int k, bool scale,
+                      hipStream_t st)
+{
+    TM_REQUIRE(xs && x && w && en2f && lds >= H && ldx >= H, "moe gather: operands");
+    if (T == 0) {
+        return 0;
+    }
+    if (elem_bytes == 2) {
+        moe_gather_kernel<__bf16><<<T * k, 256, 0, st>>>((__bf16*)xs, lds, (const __bf16*)x, ldx, w, en2f, T, H, k, scale);
+    }
+    else {
+        moe_gather_kernel<float><<<T * k, 256, 0, st>>>((float*)xs, lds, (const float*)x, ldx, w, en2f, T, H, k, scale);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+// resid[t] += gate(t) * sum_j (weighted ? w[t][j] : 1) * y[en2f[j][t]], gate(t)[i] = sigmoid(gate[t][i] + gate_bias[i]) (gate == nullptr: 1)
+__global__ void moe_combine_f32_kernel(float* __restrict__ resid, const float* __restrict__ y, const float* __restrict__ w, const int* __restrict__ en2f,
+                                       const float* __restrict__ gate, int ldg, const float* __restrict__ gate_bias, int Tn, int H, int k, int weighted)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)Tn * H) {
+        return;
+    }
+    const int t = (int)(i / H), c = (int)(i % H);
+    float     s = 0.f;
+    for (int j = 0; j < k; ++j) {
+        const float v = y[(size_t)en2f[(size_t)j * Tn + t] * H + c];
+        s += weighted ? w[(size_t)t * k + j] * v : v;
+    }
+    if (gate) {
+        s = s / (1.f + expf(-(gate[(size_t)t * ldg + c] + gate_bias[c])));
+    }
+    resid[i] += s;
+}
+
+int launch_moe_combine_f32(float* resid, const float* y, const float* w, const int* en2f, const float* gate, int ldg, const float* gate_bias, int T,
+                           int H, int k, bool weighted, hipStream_t st)
+{
+    TM_REQUIRE(resid && y && w && en2f && (!gate || (gate_bias && ldg >= H)), "moe combine: operands");
+    const size_t total = (size_t)T * H;
+    if (total == 0) {
+        return 0;
+    }
+    moe_combine_f32_kernel<<<(total + 255) / 256, 256, 0, st>>>(resid, y, w, en2f, gate, ldg, gate_bias, T, H, k, weighted);
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
 }  // namespace tmk

@@ -340,19 +340,36 @@ inline uint64_t* gemm_trace_for(size_t workgroups, const char* tag = "", int gx 
 
 // ---- gemm_dense.hip: unquantised linears, W stored [N][K]; bf16 on the matrix cores or true fp32 ------------------------------
 enum { kDenseBf16 = 0, kDenseF32 = 1 };
-// epilogues: y = acc (activation type) | y = relu(acc)^2 | y_f32 += alpha * acc (residual stream) | y_f32 = alpha * acc
-enum { kDenseStore = 0, kDenseRelu2 = 1, kDenseResidAdd = 2, kDenseScaleF32 = 3 };
+// epilogues: y = acc (activation type) | y = relu(acc)^2 | y_f32 += alpha * acc (residual stream) | y_f32 = alpha * acc |
+// y_f32 = acc + bias[n] | y_f32 += sigmoid(gate[m][n] + gate_bias[n]) * acc (gated residual sum)
+enum { kDenseStore = 0, kDenseRelu2 = 1, kDenseResidAdd = 2, kDenseScaleF32 = 3, kDenseBiasF32 = 4, kDenseResidGate = 5 };
 struct DenseWeight {
     int    K = 0, N = 0, Kp = 0, Np = 0;  // Kp = K rounded up to 32, Np = N rounded up to 128: zero-padded image [Np][Kp]
     int    dtype = kDenseBf16;
+    int    count = 1;                     // images of the same size behind each other (heads, experts)
     void*  w     = nullptr;
     size_t bytes = 0;
 };
-int  dense_weight_alloc(DenseWeight& d, int K, int N, int dtype, hipStream_t st);
+// one launch: the epilogue with its operands, and the items of a batched launch
+struct DenseCall {
+    int          epi   = kDenseStore;
+    float        alpha = 1.f;
+    const float* bias  = nullptr;       // kDenseBiasF32: [N]
+    const float* gate  = nullptr;       // kDenseResidGate: gate logits [M][ldg] and their bias [N]
+    const float* gate_bias = nullptr;
+    int          ldg   = 0;
+    int          count = 1;             // items; item g uses image g, x column g * x_col_stride, y column g * y_col_stride ...
+    int          x_col_stride = 0, y_col_stride = 0;
+    const int*   row_offsets = nullptr; // ... and, when set, the rows [row_offsets[g], row_offsets[g + 1]) of x and y (device, [count + 1])
+    size_t       w_stride = 0;          // (set by the launcher)
+};
+int  dense_weight_alloc(DenseWeight& d, int K, int N, int dtype, hipStream_t st, int count = 1);
 // rows x cols bf16 block (checkpoint orientation [out][in]) -> image rows [row0, row0 + rows), columns [col0, col0 + cols):
-// concatenation along N fuses projections of one input, along K projections that are summed
-int  dense_weight_place(DenseWeight& d, int row0, int col0, const void* src_bf16, int rows, int cols, hipStream_t st);
+// concatenation along N fuses projections of one input, along K projections that are summed.  transpose: the block is [in][out]
+int  dense_weight_place(DenseWeight& d, int row0, int col0, const void* src_bf16, int rows, int cols, hipStream_t st, int item = 0,
+                        bool transpose = false);
 void dense_weight_free(DenseWeight& d);
+int  launch_dense_call(const DenseWeight& d, const void* x, int ldx, void* y, int ldy, int M, DenseCall call, hipStream_t st);
 // x [M][ldx] (ldx >= Kp, pad columns finite), y [M][ldy]; x / y element type = the weight's dtype unless the epilogue says fp32
 int  launch_dense_linear(const DenseWeight& d, const void* x, int ldx, void* y, int ldy, int M, int epi, float alpha, hipStream_t st);
 
@@ -372,6 +389,12 @@ struct GeneralAttnParams {
     int             q_heads = 0, kv_heads = 0, dim = 0, vdim = 0;
     float           scale = 1.f, softcap = 0.f, qtemp_coef = 0.f, qtemp_every = 1.f;
     const float*    sink = nullptr;      // [q_heads] or nullptr
+    const float*    dist_r1 = nullptr;   // [q_heads] or nullptr: score -= r1 * ln(1 + r2 * (position - key position))
+    const float*    dist_r2 = nullptr;
+    int             chunk = 0;           // > 0: a row sees the keys of its own chunk of positions only (key >= floor(pos / chunk) * chunk)
+    const float*    out_gate = nullptr;  // [rows][ld_gate] or nullptr: head h of row t is multiplied by sigmoid(out_gate[t][h])
+    int             ld_gate = 0;
+    int             out_head_stride = 0; // > 0: head h of an output row starts at h * out_head_stride instead of h * vdim
     int             splits = 1;
     float*          partial_o = nullptr;   // [rows][q_heads][splits][vdim]
     float*          partial_ml = nullptr;  // [rows][q_heads][splits][2]
@@ -403,6 +426,25 @@ int launch_embedding_f32(float* out, const void* table, int table_elem_bytes, co
 int launch_rows_prepare(int* row_seq, int* row_pos, const int* cu_q, const int* k_len, int nseq, int rows, hipStream_t st);
 // keys / values of the new rows -> paged cache.  qkv [rows][ld]: keys at column k_col ([kv_heads][dim]), values at v_col ([kv_heads][vdim])
 int launch_kv_store_general(const void* qkv, int ld, int k_col, int v_col, const GeneralAttnParams& layout, hipStream_t st);
+// the same from the fp32 output of a fused projection, with optional unit-RMS scaling per head of queries + keys / of values (no weight);
+// queries -> q_out [rows][ldq] in the cache's element type
+int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col, void* q_out, int ldq, bool qk_norm, bool v_norm, float eps,
+                     const GeneralAttnParams& layout, hipStream_t st);
+// latent attention (layout: one key head, dim = C + R, vdim = C): normed latent vector + rotated shared key part -> cache; unrotated query
+// parts -> q_plain (head h at h * plain_stride), rotated query parts -> q_full[h * (C + R) + C ...]
+int launch_latent_prep(const float* proj, int ld, int q_col, int dkv_col, void* q_plain, int ldp, int plain_stride, void* q_full, int ldq,
+                       const float* c_norm_w, const float* inv_freq, int D, int R, int C, float eps, const GeneralAttnParams& layout,
+                       hipStream_t st);
+// out[m][i] = act(gu[m][i]) * gu[m][up_col + i] (act: TM_ACT_*), out bf16 | fp32
+int launch_act_mul(void* out, int ldo, int out_elem_bytes, const float* gu, int ld, int up_col, int M, int n, int act, hipStream_t st);
+// out[m] = [a[m] | b[m]] (a, b fp32 [M][H]) in bf16 | fp32
+int launch_concat2(void* out, int ldo, int out_elem_bytes, const float* a, const float* b, int M, int H, hipStream_t st);
+// mixture of experts on the fp32 stream: sigmoid router top-k from fp32 logits; gather (optionally scaled) rows in expert order; gated sum
+int launch_moe_topk_sigmoid(int* ids, float* w, const float* logits, int ld, int T, int E, int k, hipStream_t st);
+int launch_moe_gather(void* xs, int lds, const void* x, int ldx, int elem_bytes, const float* w, const int* en2f, int T, int H, int k, bool scale,
+                      hipStream_t st);
+int launch_moe_combine_f32(float* resid, const float* y, const float* w, const int* en2f, const float* gate, int ldg, const float* gate_bias, int T,
+                           int H, int k, bool weighted, hipStream_t st);
 // fp32 [n][V] -> fp16 [n][ld] (the sampler's logits rows)
 int launch_f32_to_f16_rows(half_t* out, int ld, const float* in, int n, int V, hipStream_t st);
 

@@ -1,7 +1,8 @@
 """Layer-list model family: decoders described layer by layer in their config.json.
 
     {"architecture": NAME, "width", "vocab", "norm": {"eps"}, "residual_mult", "logit_scale",
-     "layers": [{"type": MIXER, "mixer": {...sizes and constants...}, "mlp": {"kind", "ff"} | null, "weights_of": j}, ...]}
+     "layers": [{"type": MIXER, "mixer": {...sizes and constants...}, "mlp": {"kind", "ff"} | null, "weights_of": j}, ...],
+     "loop": {"start", "stop", "times"}}
 
 `FAMILIES` maps an architecture name to the reader that turns such a config into a `LayeredConfig` (the native engine's
 tm_layered_config).  Weights are one `model.safetensors` of bf16 tensors, stored [out, in] under the names the engine's slots carry
@@ -24,9 +25,9 @@ import numpy as np
 from .. import _ffi
 from .engine import Engine
 
-MIXER_ATTENTION = 1
-MLP_NONE, MLP_DENSE = 0, 1
-ACT_RELU2 = 0
+MIXER_ATTENTION, MIXER_LATENT = 1, 2
+MLP_NONE, MLP_DENSE, MLP_GATED, MLP_MOE = 0, 1, 2, 3
+ACT_RELU2, ACT_GELU_TANH, ACT_SILU = 0, 1, 2
 DTYPES = {'bfloat16': 0, 'bf16': 0, 'float32': 1, 'f32': 1}
 
 
@@ -46,6 +47,19 @@ class LayerSpec:
     mlp: int = MLP_NONE
     ff: int = 0
     act: int = ACT_RELU2
+    one_norm: bool = False        # both sublayers read norm1(x)
+    resid_gate: bool = False      # each sublayer's result times sigmoid(rg_i h + b_i)
+    loop_pass: int = -1           # >= 0: this layer run opens that pass of the loop
+    qk_unit_norm: bool = False    # queries and keys scaled to unit RMS per head
+    v_unit_norm: bool = False
+    dist_bias: bool = False       # score -= r1 * ln(1 + r2 * distance)
+    out_gate: bool = False        # a sigmoid gate per head on the attention output
+    chunk: int = 0                # > 0: keys are visible inside the query's chunk of positions only
+    kv_rank: int = 0              # latent attention: size of the cached latent vector
+    rot_dim: int = 0              # ... and of the rotated query / key part
+    rot_base: float = 10000.0
+    experts: int = 0
+    top: int = 0
 
 
 @dataclass
@@ -60,23 +74,36 @@ class LayeredConfig:
     logit_scale: float = 1.0
     eos_token_id: int | None = None
     max_position_embeddings: int = 8192
+    loop_times: int = 0           # > 0: tensors loop.in / loop.step exist
+    names: list = field(default_factory=list)   # tensor prefix of every layer run with tensors of its own ('' -> 'l<index>.')
 
     def native(self, dtype: str):
         """(tm_layered_config, keep-alive array)"""
         arr = (_ffi.LayerSpec * len(self.layers))(*[
             _ffi.LayerSpec(s.mixer, s.weights_of, s.heads, s.kv_heads, s.dim, s.vdim, s.scale, s.softcap, s.qtemp_coef, s.qtemp_every,
-                           int(s.sink), s.mlp, s.ff, s.act) for s in self.layers])
+                           int(s.sink), s.mlp, s.ff, s.act, int(s.one_norm), int(s.resid_gate), s.loop_pass, int(s.qk_unit_norm),
+                           int(s.v_unit_norm), int(s.dist_bias), int(s.out_gate), s.chunk, s.kv_rank, s.rot_dim, s.rot_base, s.experts, s.top)
+            for s in self.layers])
         return _ffi.LayeredConfig(self.width, self.vocab, len(self.layers), arr, self.norm_eps, self.norm_offset, self.residual_mult,
-                                  self.logit_scale, DTYPES[dtype]), arr
+                                  self.logit_scale, DTYPES[dtype], self.loop_times), arr
+
+    def tensor_name(self, run: int, leaf: str) -> str:
+        """checkpoint name of tensor `leaf` of layer run `run` (the engine's slots count layer RUNS; a looped model's file counts layers)"""
+        return (self.names[run] if self.names else f'l{run}.') + leaf
 
     def tensor_shapes(self) -> dict:
         """{tensor name: shape} a checkpoint of this config holds"""
         W, out = self.width, {'embed': (self.vocab, self.width), 'final.norm': (self.width,), 'head': (self.vocab, self.width)}
+        if self.loop_times > 0:
+            out['loop.in'], out['loop.step'] = (W, 2 * W), (self.loop_times, W)
         for i, s in enumerate(self.layers):
             if s.weights_of >= 0:
                 continue
             p = f'l{i}.'
             out[p + 'norm1'] = (W,)
+            if s.mixer == MIXER_LATENT or s.one_norm:
+                out.update(_wide_shapes(p, s, W))
+                continue
             out[p + 'mix.q'], out[p + 'mix.k'] = (s.heads * s.dim, W), (s.kv_heads * s.dim, W)
             out[p + 'mix.v'], out[p + 'mix.o'] = (s.kv_heads * s.vdim, W), (W, s.heads * s.vdim)
             if s.sink:
@@ -84,6 +111,92 @@ class LayeredConfig:
             if s.mlp:
                 out[p + 'norm2'], out[p + 'mlp.up'], out[p + 'mlp.down'] = (W,), (s.ff, W), (W, s.ff)
         return out
+
+
+def _wide_shapes(p: str, s: LayerSpec, W: int) -> dict:
+    """tensors of a block with one norm: the mixer's, the residual gates', the feed-forward's"""
+    out = {p + 'mix.o': (W, s.heads * s.vdim)}
+    if s.mixer == MIXER_LATENT:
+        out[p + 'mix.q'] = (s.heads * (s.dim + s.rot_dim), W)
+        out[p + 'mix.dkv'], out[p + 'mix.dkv.norm'] = (s.kv_rank + s.rot_dim, W), (s.kv_rank,)
+        out[p + 'mix.uk'], out[p + 'mix.uv'] = (s.heads * s.dim, s.kv_rank), (s.heads * s.vdim, s.kv_rank)
+    else:
+        out[p + 'mix.q'], out[p + 'mix.k'], out[p + 'mix.v'] = (s.heads * s.dim, W), (s.kv_heads * s.dim, W), (s.kv_heads * s.vdim, W)
+        if s.out_gate:
+            out[p + 'mix.g'] = (s.heads, W)
+    if s.dist_bias:
+        out[p + 'mix.r1'], out[p + 'mix.r2'] = (s.heads,), (s.heads,)
+    if s.sink:
+        out[p + 'mix.sink'] = (s.heads,)
+    if s.resid_gate:
+        out[p + 'rg1'], out[p + 'rg1.b'] = (W, W), (W,)
+        if s.mlp:
+            out[p + 'rg2'], out[p + 'rg2.b'] = (W, W), (W,)
+    if s.mlp == MLP_GATED:
+        out[p + 'mlp.gate'], out[p + 'mlp.up'], out[p + 'mlp.down'] = (s.ff, W), (s.ff, W), (W, s.ff)
+    elif s.mlp == MLP_MOE:
+        out[p + 'mlp.router'] = (s.experts, W)
+        for e in range(s.experts):
+            out[p + f'mlp.e{e}.gate'], out[p + f'mlp.e{e}.up'], out[p + f'mlp.e{e}.down'] = (s.ff, W), (s.ff, W), (W, s.ff)
+    return out
+
+
+def _bedenex_layer(i: int, L: dict) -> LayerSpec:
+    m, mlp = L['mixer'], L.get('mlp')
+    s = LayerSpec(heads=int(m['heads']), dim=int(m['dim']), vdim=int(m['vdim']), scale=float(m['scale']), one_norm=True, resid_gate=True)
+    if L['type'] == 'attention':
+        s.mixer, s.kv_heads = MIXER_ATTENTION, int(m['kv_heads'])
+        s.qk_unit_norm = s.v_unit_norm = s.dist_bias = s.out_gate = True
+        s.chunk = int((m.get('mask') or {}).get('size') or 0)
+    elif L['type'] == 'latent_attention':
+        s.mixer, s.kv_heads, s.sink = MIXER_LATENT, 1, True
+        s.kv_rank, s.rot_dim, s.rot_base = int(m['kv_rank']), int(m['rot_dim']), float(m['rot']['base'])
+        if int(m['rot'].get('dims', s.rot_dim)) != s.rot_dim:
+            raise NotImplementedError(f'layer {i}: the whole rotated part turns (rot.dims == rot_dim)')
+    else:
+        raise NotImplementedError(f'layer {i}: mixer {L["type"]!r}')
+    if mlp is None:
+        return s
+    if mlp.get('kind') == 'dense':
+        s.mlp, s.ff, s.act = MLP_GATED, int(mlp['ff']), ACT_GELU_TANH
+    elif mlp.get('kind') == 'moe':
+        s.mlp, s.ff, s.act = MLP_MOE, int(mlp['expert']['ff']), ACT_SILU
+        s.experts, s.top = int(mlp['router']['experts']), int(mlp['router']['top'])
+    else:
+        raise NotImplementedError(f'layer {i}: feed-forward kind {mlp.get("kind")!r}')
+    return s
+
+
+def _bedenex(c: dict) -> LayeredConfig:
+    """Bedenex: blocks x += sigmoid(rg1 h + b1) * mixer(h) + sigmoid(rg2 h + b2) * ff(h) with ONE norm h of the stream.  Mixers: grouped-query
+    attention without rotation (unit-RMS queries, keys and values per head, a logarithmic distance penalty, keys visible inside the
+    query's chunk of positions, a sigmoid gate per head on the output) and latent attention (one normed latent vector and one rotated key
+    part cached per token, a sink logit per head).  Feed-forwards: gated GELU, or a sigmoid-routed mixture of gated SiLU experts whose
+    scores scale the experts' inputs.  A range of layers may run several times in a row on the same weights (every run has its own cache);
+    each pass starts from loop.in [x | embedding output] + loop.step[pass]."""
+    import copy
+    own = [_bedenex_layer(i, L) for i, L in enumerate(c['layers'])]
+    loop = c.get('loop') or {}
+    start, stop, times = int(loop.get('start', 0)), int(loop.get('stop', 0)), int(loop.get('times', 0))
+    if stop <= start or times < 1:
+        start = stop = times = 0
+    runs, names = [], []
+    first_run = {}      # layer -> its first run (the one that owns the tensors)
+    order = list(range(start)) + [i for _ in range(times) for i in range(start, stop)] + list(range(stop, len(own)))
+    seen_pass = 0
+    for i in order:
+        s = copy.copy(own[i])
+        if times and i == start:
+            s.loop_pass, seen_pass = seen_pass, seen_pass + 1
+        if i in first_run:
+            s.weights_of = first_run[i]
+        else:
+            first_run[i] = len(runs)
+        runs.append(s)
+        names.append(f'l{i}.')
+    return LayeredConfig(arch='Bedenex', width=int(c['width']), vocab=int(c['vocab']), layers=runs, norm_eps=float(c['norm']['eps']),
+                         norm_offset=0.0, residual_mult=1.0, logit_scale=1.0, eos_token_id=c.get('eos_token_id'), loop_times=times,
+                         names=names)
 
 
 def _fokonex(c: dict) -> LayeredConfig:
@@ -113,7 +226,7 @@ def _fokonex(c: dict) -> LayeredConfig:
                          logit_scale=float(c['logit_scale']), eos_token_id=c.get('eos_token_id'))
 
 
-FAMILIES = {'Fokonex': _fokonex}
+FAMILIES = {'Fokonex': _fokonex, 'Bedenex': _bedenex}
 
 
 def is_layered(model_path: str) -> bool:
@@ -172,11 +285,16 @@ class LayeredEngine(Engine):
     def load_checkpoint(self, model_path: str):
         tensors = read_safetensors(os.path.join(model_path, 'model.safetensors'))
         for name, shape in self.model.tensor_shapes().items():
+            slot = name
+            if self.model.names and name[0] == 'l' and name[1].isdigit():   # the engine's slot counts layer runs, the file counts layers
+                run, leaf = name[1:].split('.', 1)
+                name = self.model.tensor_name(int(run), leaf)
             if name not in tensors:
                 raise KeyError(f'{model_path}: tensor {name} is missing')
             dt, shp, data = tensors[name]
             if dt != 'BF16' or tuple(shp) != tuple(shape):
                 raise ValueError(f'{name}: {dt} {shp} in the file, the config says BF16 {shape}')
+            name = slot
             buf = np.frombuffer(data, np.uint8)
             _ffi.check(self._lib.tm_engine_weight_copy(self._h, name.encode(), buf.ctypes.data, buf.nbytes))
         _ffi.check(self._lib.tm_engine_process_weights(self._h))
