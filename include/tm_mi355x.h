@@ -608,6 +608,13 @@ typedef struct tm_general_attn {
     int             ldkv, k_col, v_col, store_kv;
     int             kernel, prefill, nseq, max_q_len;
     const int *     cu_q, *k_len;
+    /* all off at 0 / NULL: score -= dist_r1[head] * ln(1 + dist_r2[head] * (position - key position)); chunk > 0: a row sees the keys of
+     * its own chunk of positions only; out_gate [rows][ld_gate] fp32: head h of row t *= sigmoid(out_gate[t][h]); out_head_stride > 0:
+     * head h of an output row starts at h * out_head_stride */
+    const float *   dist_r1, *dist_r2;
+    int             chunk;
+    const float*    out_gate;
+    int             ld_gate, out_head_stride;
 } tm_general_attn;
 size_t tm_general_attention_workspace(int rows, int q_heads, int vdim, int splits);
 int    tm_general_attention(const tm_general_attn* a, tm_stream_t st);

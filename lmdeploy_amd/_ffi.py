@@ -95,7 +95,8 @@ class GeneralAttn(C.Structure):
                 ('scale', c_float), ('softcap', c_float), ('qtemp_coef', c_float), ('qtemp_every', c_float), ('sink', c_void_p),
                 ('splits', c_int), ('workspace', c_void_p), ('kv', c_void_p), ('ldkv', c_int), ('k_col', c_int), ('v_col', c_int),
                 ('store_kv', c_int), ('kernel', c_int), ('prefill', c_int), ('nseq', c_int), ('max_q_len', c_int), ('cu_q', c_void_p),
-                ('k_len', c_void_p)]
+                ('k_len', c_void_p), ('dist_r1', c_void_p), ('dist_r2', c_void_p), ('chunk', c_int), ('out_gate', c_void_p),
+                ('ld_gate', c_int), ('out_head_stride', c_int)]
 
 
 # name -> (restype, argtypes); every int-returning function is a tm_status

@@ -6,6 +6,10 @@ in its sequence (from 0).  Weights are stored [out, in] and applied as h @ w.T.
 """
 from __future__ import annotations
 
+import json
+import os
+import struct
+
 import numpy as np
 
 
@@ -107,10 +111,17 @@ def dense_ff(h, t):
     return (gelu_tanh(h @ t['gate'].T) * (h @ t['up'].T)) @ t['down'].T
 
 
+ROUTER_GAPS = []      # smallest gap between the last chosen and the first rejected router logit of every moe_ff call since it was cleared
+
+
 def moe_ff(h, t, mlp):
     """sigmoid router; the `top` best experts of a token (ties: the lower index); the score scales the expert's INPUT"""
     E, top = mlp['router']['experts'], mlp['router']['top']
-    score = sigmoid(h @ t['router'].T)
+    z = h @ t['router'].T
+    score = sigmoid(z)
+    if top < E:
+        zs = np.sort(z, axis=-1)
+        ROUTER_GAPS.append(float((zs[:, E - top] - zs[:, E - top - 1]).min()))
     out = np.zeros((h.shape[0], t['e0.down'].shape[0]))
     for n in range(h.shape[0]):
         for e in np.argsort(-score[n], kind='stable')[:top]:
@@ -155,6 +166,14 @@ def layer_runs(cfg):
     return runs + [(i, None) for i in range(loop['stop'], n)]
 
 
+def router_gap(cfg, tensors, requests):
+    """the closest call any router makes over these token lists (logit units): reduced-precision runs may route a closer one differently"""
+    ROUTER_GAPS.clear()
+    for t in requests:
+        forward(cfg, tensors, t)
+    return min(ROUTER_GAPS) if ROUTER_GAPS else np.inf
+
+
 def forward(cfg, tensors, tokens, want_layers=False):
     """tensors: {name: float64 array}; -> logits [T, vocab] (and the residual stream behind every layer run)"""
     eps = cfg['norm']['eps']
@@ -167,3 +186,119 @@ def forward(cfg, tensors, tokens, want_layers=False):
         trail.append(x)
     logits = rms_norm(x, tensors['final.norm'], eps) @ tensors['head'].T
     return (logits, np.stack(trail)) if want_layers else logits
+
+
+# ---- the tests' own models -----------------------------------------------------------------------------------------------------------
+def bf16_round(x):
+    """float64 values rounded to the nearest bfloat16 (ties to even), as float64"""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    u = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return u.astype(np.uint32).view(np.float32).astype(np.float64)
+
+
+def bf16_bits(x):
+    return (np.ascontiguousarray(bf16_round(x), np.float32).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def attention_layer(heads, kv_heads, dim, vdim, scale, chunk, mlp=None):
+    m = {'heads': heads, 'kv_heads': kv_heads, 'dim': dim, 'vdim': vdim, 'scale': scale}
+    if chunk:
+        m['mask'] = {'size': chunk}
+    return {'type': 'attention', 'mixer': m, 'mlp': mlp}
+
+
+def latent_layer(heads, dim, rot_dim, vdim, kv_rank, scale, base=10000.0, mlp=None):
+    return {'type': 'latent_attention', 'mlp': mlp,
+            'mixer': {'heads': heads, 'dim': dim, 'rot_dim': rot_dim, 'vdim': vdim, 'kv_rank': kv_rank, 'scale': scale,
+                      'rot': {'base': base, 'dims': rot_dim}}}
+
+
+def dense(ff):
+    return {'kind': 'dense', 'ff': ff}
+
+
+def moe(experts, top, ff):
+    return {'kind': 'moe', 'expert': {'ff': ff}, 'router': {'experts': experts, 'top': top}}
+
+
+def make_config(width, vocab, layers, loop=None, eps=1e-5):
+    c = {'architecture': 'Bedenex', 'width': width, 'vocab': vocab, 'layers': layers, 'norm': {'eps': eps}}
+    if loop:
+        c['loop'] = {'start': loop[0], 'stop': loop[1], 'times': loop[2]}
+    return c
+
+
+def make_weights(cfg, seed, sink=3.0):
+    """bf16-representable float64 tensors under the checkpoint's names.  Projections N(0, 1 / inputs); sinks around `sink` so that a
+    forgotten sink moves every latent layer's output; distance numbers positive; gate biases around zero"""
+    rng = np.random.default_rng(seed)
+    W, w = cfg['width'], {}
+
+    def mat(n_out, n_in, gain=1.0):
+        return bf16_round(rng.normal(0, gain / np.sqrt(n_in), (n_out, n_in)))
+
+    def vec(n, mean, std):
+        return bf16_round(rng.normal(mean, std, n))
+
+    w['embed'] = bf16_round(rng.normal(0, 1, (cfg['vocab'], W)))
+    w['head'], w['final.norm'] = mat(cfg['vocab'], W), vec(W, 1.0, 0.2)
+    loop = cfg.get('loop')
+    if loop:
+        w['loop.in'], w['loop.step'] = mat(W, 2 * W), bf16_round(rng.normal(0, 0.3, (loop['times'], W)))
+    for i, L in enumerate(cfg['layers']):
+        p, m = f'l{i}.', L['mixer']
+        H, D, V = m['heads'], m['dim'], m['vdim']
+        w[p + 'norm1'] = vec(W, 1.0, 0.2)
+        w[p + 'rg1'], w[p + 'rg1.b'] = mat(W, W), vec(W, 0.0, 0.5)
+        w[p + 'mix.o'] = mat(W, H * V)
+        if L['type'] == 'attention':
+            G = m['kv_heads']
+            w[p + 'mix.q'], w[p + 'mix.k'], w[p + 'mix.v'] = mat(H * D, W), mat(G * D, W), mat(G * V, W)
+            w[p + 'mix.g'] = mat(H, W)
+            w[p + 'mix.r1'], w[p + 'mix.r2'] = np.abs(vec(H, 1.0, 0.6)), np.abs(vec(H, 0.3, 0.15))
+        else:
+            R, C = m['rot_dim'], m['kv_rank']
+            w[p + 'mix.q'], w[p + 'mix.dkv'] = mat(H * (D + R), W, 2.0), mat(C + R, W, 2.0)
+            w[p + 'mix.dkv.norm'] = vec(C, 1.0, 0.2)
+            w[p + 'mix.uk'], w[p + 'mix.uv'] = mat(H * D, C, 2.0), mat(H * V, C)
+            w[p + 'mix.sink'] = vec(H, sink, 1.0)
+        mlp = L.get('mlp')
+        if mlp is None:
+            continue
+        w[p + 'rg2'], w[p + 'rg2.b'] = mat(W, W), vec(W, 0.0, 0.5)
+        if mlp['kind'] == 'dense':
+            w[p + 'mlp.gate'], w[p + 'mlp.up'], w[p + 'mlp.down'] = mat(mlp['ff'], W, 2.0), mat(mlp['ff'], W), mat(W, mlp['ff'])
+        else:
+            w[p + 'mlp.router'] = mat(mlp['router']['experts'], W, 6.0)
+            ff = mlp['expert']['ff']
+            for e in range(mlp['router']['experts']):
+                w[p + f'mlp.e{e}.gate'], w[p + f'mlp.e{e}.up'], w[p + f'mlp.e{e}.down'] = mat(ff, W, 3.0), mat(ff, W, 2.0), mat(W, ff)
+    return w
+
+
+def write_checkpoint(folder, cfg, w):
+    """config.json + model.safetensors (8-byte length, JSON header, bf16 data), written by hand"""
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, 'config.json'), 'w') as f:
+        json.dump(cfg, f)
+    header, blobs, off = {}, [], 0
+    for name in sorted(w):
+        b = bf16_bits(w[name]).astype('<u2').tobytes()
+        header[name] = {'dtype': 'BF16', 'shape': list(np.shape(w[name])), 'data_offsets': [off, off + len(b)]}
+        blobs.append(b)
+        off += len(b)
+    hj = json.dumps(header).encode()
+    with open(os.path.join(folder, 'model.safetensors'), 'wb') as f:
+        f.write(struct.pack('<Q', len(hj)) + hj + b''.join(blobs))
+
+
+def greedy(cfg, w, prompt, n_new):
+    """-> (tokens, margins): arg-max continuation and the top-1 / top-2 logit gap of every step"""
+    toks, out, margins = list(prompt), [], []
+    for _ in range(n_new):
+        lg = forward(cfg, w, toks)[-1]
+        top = np.sort(lg)[-2:]
+        out.append(int(lg.argmax()))
+        margins.append(float(top[1] - top[0]))
+        toks.append(out[-1])
+    return out, margins
