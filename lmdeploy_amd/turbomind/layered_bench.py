@@ -5,6 +5,10 @@ feed-forward's three).  Random weights; both engines run their own static-batch 
 
 Per kernel category of an eager decode step the table also gives the fraction of the HBM roofline (bytes the category must move /
 8 TB/s / measured time) for both, and their ratio: the figure the two designs' like kernels are compared by.
+
+`bench.py --layered --layered-design bedenex`: the same for Bedenex blocks (chunked attention with unit norms, distance penalty and output
+gate; latent attention; gated residuals; gated-GELU and routed-expert feed-forwards; a looped range of layers) beside the closest
+model the engine serves, the Fokonex blocks above, at equal width, heads, layer count, vocabulary and active feed-forward parameters.
 """
 from __future__ import annotations
 
@@ -31,6 +35,53 @@ def _fokonex_engine(s, batch, session_len, max_prefill):
     eng.init_synthetic(seed=1)
     eng.start()
     return eng
+
+
+BEDENEX = dict(chunk=2048, latent_dim=64, rot_dim=64, kv_rank=192, experts=8, top=2)
+
+
+def bedenex_config(s) -> dict:
+    """config.json of the benchmark model: [attention + dense, attention + experts, latent + dense, latent + experts] repeated, the middle
+    layers inside a loop that runs once.  Experts of half the dense size, two per token: the active parameters equal the dense block's"""
+    b = BEDENEX
+    att = {'heads': s['heads'], 'kv_heads': s['kv_heads'], 'dim': 128, 'vdim': 128, 'scale': 128 ** -0.5, 'mask': {'size': b['chunk']}}
+    lat = {'heads': s['heads'], 'dim': b['latent_dim'], 'rot_dim': b['rot_dim'], 'vdim': 128, 'kv_rank': b['kv_rank'], 'scale': 128 ** -0.5,
+           'rot': {'base': 10000.0, 'dims': b['rot_dim']}}
+    dense = {'kind': 'dense', 'ff': s['inter']}
+    moe = {'kind': 'moe', 'expert': {'ff': s['inter'] // 2}, 'router': {'experts': b['experts'], 'top': b['top']}}
+    four = [{'type': 'attention', 'mixer': att, 'mlp': dense}, {'type': 'attention', 'mixer': att, 'mlp': moe},
+            {'type': 'latent_attention', 'mixer': lat, 'mlp': dense}, {'type': 'latent_attention', 'mixer': lat, 'mlp': moe}]
+    n = s['layers']
+    return {'architecture': 'Bedenex', 'width': s['width'], 'vocab': s['vocab'], 'norm': {'eps': 1e-5},
+            'layers': [four[i % 4] for i in range(n)], 'loop': {'start': n // 4, 'stop': n - n // 4, 'times': 1}}
+
+
+def _bedenex_engine(s, batch, session_len, max_prefill):
+    from . import layered
+    cfg = layered.FAMILIES['Bedenex'](bedenex_config(s))
+    eng = layered.LayeredEngine(cfg, dtype='bfloat16', max_batch_size=batch, session_len=session_len, max_prefill_token_num=max_prefill)
+    eng.init_synthetic(seed=1)
+    eng.start()
+    return eng
+
+
+def _bedenex_decode_bytes(s, batch, ctx):
+    """bytes each category of ONE decode step must move: every weight that takes part once (all experts: batch x top pairs reach each of
+    them), the cache entries a row sees once per sequence; activations are noise beside them"""
+    b, W, H, G, I, V = BEDENEX, s['width'], s['heads'], s['kv_heads'], s['inter'], s['vocab']
+    C, R, D = b['kv_rank'], b['rot_dim'], b['latent_dim']
+    out = dict(gemm_qkv=0, attention=0, gemm_o=2 * W * 2 * W, gemm_gate_up=0, gemm_down=0, lm_head=2 * W * V)
+    for i in range(s['layers']):
+        latent, moe = i % 4 >= 2, i % 2 == 1
+        n_proj = (H * (D + R) + C + R if latent else (H + 2 * G) * 128 + H) + 2 * W + (b['experts'] if moe else 0)
+        out['gemm_qkv'] += 2 * W * n_proj + (2 * H * D * C if latent else 0)
+        # the latent cache holds the latent vector twice: inside the key rows and, transposed, as the value rows
+        out['attention'] += 2 * batch * ((C + R + C) * ctx if latent else 2 * G * 128 * min(ctx, b['chunk'] // 2 if ctx > b['chunk'] else ctx))
+        out['gemm_o'] += 2 * W * H * 128 + (2 * H * 128 * C if latent else 0)
+        ff = b['experts'] * (I // 2) if moe else I
+        out['gemm_gate_up'] += 2 * W * 2 * ff
+        out['gemm_down'] += 2 * W * ff
+    return out
 
 
 def _llama_engine(s, batch, session_len, max_prefill):
@@ -90,22 +141,29 @@ def _decode_bytes(s, batch, ctx, fokonex: bool):
     return b
 
 
-def run(steps: int, warmup: int, batch: int, prompt_len: int, sizes=None) -> dict:
+def run(steps: int, warmup: int, batch: int, prompt_len: int, sizes=None, design: str = 'fokonex') -> dict:
     res = {}
+    pair = (('fokonex_bf16', _fokonex_engine), ('llama_f16', _llama_engine)) if design == 'fokonex' else \
+        (('bedenex_bf16', _bedenex_engine), ('fokonex_bf16', _fokonex_engine))
     for name in (sizes or SIZES):
         s = SIZES[name]
         session_len = prompt_len + steps + warmup + 64
         prefill_seqs = max(1, 8192 // prompt_len)
         row = {}
-        for kind, make in (('fokonex_bf16', _fokonex_engine), ('llama_f16', _llama_engine)):
+        for kind, make in pair:
             eng = make(s, batch, session_len, 8192)
             m = _measure(eng, s['vocab'], batch, prompt_len, steps, warmup, prefill_seqs)
-            need = _decode_bytes(s, batch, prompt_len + warmup + steps // 2, kind == 'fokonex_bf16')
+            ctx = prompt_len + warmup + steps // 2
+            need = _bedenex_decode_bytes(s, batch, ctx) if kind == 'bedenex_bf16' else _decode_bytes(s, batch, ctx, kind == 'fokonex_bf16')
             m['decode_hbm_roofline_fraction'] = {k: round(need[k] / HBM_BYTES_PER_S / (m['decode_categories_ms'][k] * 1e-3), 4)
                                                  for k in need if m['decode_categories_ms'].get(k)}
             eng.close()
             row[kind] = m
-        f, l = row['fokonex_bf16'], row['llama_f16']
+        f, l = row[pair[0][0]], row[pair[1][0]]
+        if design != 'fokonex':   # how much farther from its roofline each category of the new design runs than the like one beside it
+            fa, fb = f['decode_hbm_roofline_fraction'], l['decode_hbm_roofline_fraction']
+            fb = dict(fb, gemm_down=fb.get('gemm_down', fb.get('gemm_o')))      # (Fokonex closes a block with ONE [o | down] product)
+            row['roofline_distance_ratio'] = {k: round(fb[k] / fa[k], 2) for k in fa if fb.get(k) and fa[k] > 0}
         row['prefill_ratio'] = round(f['prefill_tokens_per_s'] / l['prefill_tokens_per_s'], 3)
         row['decode_ratio'] = round(f['decode_tokens_per_s'] / l['decode_tokens_per_s'], 3)
         res[name] = row
