@@ -348,13 +348,14 @@ def main():
     ap.add_argument('--cpu-config0', action='store_true',
                     help='BASELINE.json configs[0] only: InternLM2-1.8B fp16 greedy decode on the host cores (oracle/cpu_baseline.py::run_config0, the '
                          'torch-CPU port of the reference\'s default-backend ops); prints its own JSON line; no GPU is touched')
+    ap.add_argument('--layered-one', action='store_true', help='with --layered: run the design itself only, not the model beside it (kernel traces)')
     args = ap.parse_args()
     if args.layered:
         from lmdeploy_amd.turbomind import layered_bench
         steps = 64 if args.steps == 512 else args.steps
         batch = 32 if args.batch == 64 else args.batch
         r = layered_bench.run(steps, args.warmup, batch, args.prompt_len, [x for x in args.layered_sizes.split(',') if x] or None,
-                              args.layered_design)
+                              args.layered_design, args.layered_one)
         first, beside = ('fokonex_bf16', 'the fp16 Llama-family engine') if args.layered_design == 'fokonex' else ('bedenex_bf16', 'Fokonex blocks')
         emit_json({'metric': f'prefill and decode tokens/sec of a {args.layered_design.capitalize()} layer-list model (bf16) beside {beside} at equal size, '
                              f'decode batch {batch}, context {args.prompt_len}', 'value': round(next(iter(r.values()))[first]['decode_tokens_per_s'], 1),

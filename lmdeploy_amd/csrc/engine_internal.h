@@ -99,12 +99,12 @@ struct LayeredModel {
     float*               final_norm = nullptr;
     int                  elem       = 2;        // bytes of an activation / cache element
     int                  ldw = 0, ldqkv = 0, ldcat = 0, ldv16 = 0;  // leading dimensions: normed rows, projections, [attention | ff], fp16 logits
-    int                  ldproj = 0, ldq = 0, ldplain = 0, ldlat = 0, ldgu = 0, ldff = 0, ld2w = 0, max_top = 0;
+    int                  ldproj = 0, ldq = 0, ldplain = 0, ldlat = 0, ldff = 0, ld2w = 0, max_top = 0;
     int                  max_logit_rows = 0;
     float*               d_res = nullptr;       // residual stream [max_tokens][width]
     void *               d_h1 = nullptr, *d_h2 = nullptr, *d_qkv = nullptr, *d_cat = nullptr, *d_hn = nullptr;
-    // wide blocks: fused projection (fp32), queries, unrotated query parts, latent attention output, [gate | up] (fp32), activations
-    float *              d_proj = nullptr, *d_gu = nullptr, *d_x0 = nullptr, *d_moe_y = nullptr, *d_topk_w = nullptr;
+    // wide blocks: fused projection (fp32), queries, unrotated query parts, latent attention output, activations
+    float *              d_proj = nullptr, *d_x0 = nullptr, *d_moe_y = nullptr, *d_topk_w = nullptr;
     void *               d_q = nullptr, *d_plain = nullptr, *d_lat = nullptr, *d_ff = nullptr, *d_xx = nullptr, *d_moe_x = nullptr;
     int *                d_topk_ids = nullptr, *d_offsets = nullptr, *d_f2n = nullptr, *d_en2f = nullptr;
     float*               d_logits_f32 = nullptr;  // [max_logit_rows][vocab]

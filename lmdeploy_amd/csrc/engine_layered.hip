@@ -19,7 +19,8 @@
 //   attention (chunk, distance penalty, sink, output gate as parameters)
 //   latent:  cat[:, head] = lat[:, head] . uv_head^T               one batched GEMM (the value expansion)
 //   x       += sigmoid(proj[rg1] + b1) * (cat . Wo^T)              GEMM with the gated-residual epilogue
-//   dense:   gu = h . [gate | up]^T (fp32); a = act(gate) * up; x += sigmoid(proj[rg2] + b2) * (a . Wdown^T)
+//   dense:   a = act(h . gate^T) * (h . up^T)  ONE GEMM over the interleaved [gate | up] image, activation in its epilogue;
+//            x += sigmoid(proj[rg2] + b2) * (a . Wdown^T)
 //   experts: router top-k -> rows sorted by expert, scaled by their score -> the same two products batched over the experts -> gated sum
 #include "engine_internal.h"
 
@@ -59,6 +60,8 @@ __global__ void iota_kernel(int* out, int n)
     }
 }
 
+static_assert(kActRelu2 == TM_ACT_RELU2 && kActGeluTanh == TM_ACT_GELU_TANH && kActSilu == TM_ACT_SILU, "activation codes");
+
 static std::string lname(int i, const char* t)
 {
     return "l" + std::to_string(i) + "." + t;
@@ -82,12 +85,12 @@ static int to_f32(tm_engine* e, const std::string& name, size_t n, float** out)
 }
 
 static int place(tm_engine* e, DenseWeight& d, int row0, int col0, const std::string& name, int rows, int cols, size_t src_row = 0, int item = 0,
-                 bool transpose = false)
+                 bool transpose = false, int half = 0)
 {
     Slot& s = e->slots[name];
     TM_REQUIRE(s.filled, "weight not loaded: " + name);
     TM_REQUIRE((int64_t)(src_row + rows) * cols * 2 <= s.bytes, "internal: weight part outside " + name);
-    return dense_weight_place(d, row0, col0, (const uint16_t*)s.dev + src_row * cols, rows, cols, e->stream, item, transpose);
+    return dense_weight_place(d, row0, col0, (const uint16_t*)s.dev + src_row * cols, rows, cols, e->stream, item, transpose, half);
 }
 
 static int process_wide_layer(tm_engine* e, int i, LmLayer& L, int dt)
@@ -142,20 +145,20 @@ static int process_wide_layer(tm_engine* e, int i, LmLayer& L, int dt)
         }
     }
     if (s.mlp == TM_MLP_GATED) {
-        TM_TRY(dense_weight_alloc(L.gu, W, 2 * s.ff, dt, e->stream));
-        TM_TRY(place(e, L.gu, 0, 0, lname(i, "mlp.gate"), s.ff, W));
-        TM_TRY(place(e, L.gu, s.ff, 0, lname(i, "mlp.up"), s.ff, W));
+        TM_TRY(dense_weight_alloc(L.gu, W, dense_pair_rows(s.ff), dt, e->stream));  // gate and up interleaved: the activation is the GEMM's epilogue
+        TM_TRY(place(e, L.gu, 0, 0, lname(i, "mlp.gate"), s.ff, W, 0, 0, false, 1));
+        TM_TRY(place(e, L.gu, 0, 0, lname(i, "mlp.up"), s.ff, W, 0, 0, false, 2));
         TM_TRY(dense_weight_alloc(L.down, s.ff, W, dt, e->stream));
         TM_TRY(place(e, L.down, 0, 0, lname(i, "mlp.down"), W, s.ff));
     }
     else if (s.mlp == TM_MLP_MOE) {
         TM_TRY(place(e, L.qkv, L.c_router, 0, lname(i, "mlp.router"), s.experts, W));
-        TM_TRY(dense_weight_alloc(L.gu, W, 2 * s.ff, dt, e->stream, s.experts));
+        TM_TRY(dense_weight_alloc(L.gu, W, dense_pair_rows(s.ff), dt, e->stream, s.experts));
         TM_TRY(dense_weight_alloc(L.down, s.ff, W, dt, e->stream, s.experts));
         for (int x = 0; x < s.experts; ++x) {
             const std::string ex = "mlp.e" + std::to_string(x) + ".";
-            TM_TRY(place(e, L.gu, 0, 0, lname(i, (ex + "gate").c_str()), s.ff, W, 0, x));
-            TM_TRY(place(e, L.gu, s.ff, 0, lname(i, (ex + "up").c_str()), s.ff, W, 0, x));
+            TM_TRY(place(e, L.gu, 0, 0, lname(i, (ex + "gate").c_str()), s.ff, W, 0, x, false, 1));
+            TM_TRY(place(e, L.gu, 0, 0, lname(i, (ex + "up").c_str()), s.ff, W, 0, x, false, 2));
             TM_TRY(place(e, L.down, 0, 0, lname(i, (ex + "down").c_str()), W, s.ff, 0, x));
         }
     }
@@ -309,7 +312,7 @@ int layered_start(tm_engine* e)
     lm.ldw      = (m.width + 31) / 32 * 32;
     int64_t off = 0;
     int     max_qkv = 8, max_cat = 32, max_vdim = 0, max_heads = 0;
-    int     max_proj = 0, max_q = 0, max_plain = 0, max_lat = 0, max_gu = 0, max_ff = 0;
+    int     max_proj = 0, max_q = 0, max_plain = 0, max_lat = 0, max_ff = 0;
     bool    any_moe = false;
     for (LmLayer& L : lm.layers) {
         L.kv_offset = off;
@@ -329,7 +332,6 @@ int layered_start(tm_engine* e)
         max_plain = std::max(max_plain, L.spec.heads * L.plain_stride);
         max_lat   = std::max(max_lat, L.spec.heads * L.lat_stride);
         if (L.spec.mlp) {
-            max_gu     = std::max(max_gu, L.gu.N);
             max_ff     = std::max(max_ff, L.down.Kp);
             lm.max_top = std::max(lm.max_top, L.spec.mlp == TM_MLP_MOE ? L.spec.top : 1);
             any_moe    = any_moe || L.spec.mlp == TM_MLP_MOE;
@@ -346,13 +348,11 @@ int layered_start(tm_engine* e)
         lm.ldq     = (max_q + 31) / 32 * 32;
         lm.ldplain = std::max(32, max_plain);
         lm.ldlat   = std::max(32, max_lat);
-        lm.ldgu    = std::max(4, (max_gu + 3) / 4 * 4);
         lm.ldff    = std::max(32, max_ff);
         TM_TRY(lm_alloc(&lm.d_proj, T * lm.ldproj, st));
         TM_TRY(lm_alloc((char**)&lm.d_q, T * lm.ldq * lm.elem, st));
         TM_TRY(lm_alloc((char**)&lm.d_plain, T * lm.ldplain * lm.elem, st));
         TM_TRY(lm_alloc((char**)&lm.d_lat, T * lm.ldlat * lm.elem, st));
-        TM_TRY(lm_alloc(&lm.d_gu, TT * lm.ldgu, st));
         TM_TRY(lm_alloc((char**)&lm.d_ff, TT * lm.ldff * lm.elem, st));
         if (any_moe) {
             TM_TRY(lm_alloc((char**)&lm.d_moe_x, TT * lm.ldw * lm.elem, st));
@@ -455,7 +455,7 @@ void layered_free(tm_engine* e)
     }
     dense_weight_free(lm.head);
     dense_weight_free(lm.loop_in);
-    for (void* p : {(void*)lm.loop_step, (void*)lm.d_proj, (void*)lm.d_gu, (void*)lm.d_x0, (void*)lm.d_moe_y, (void*)lm.d_topk_w, lm.d_q, lm.d_plain, lm.d_lat,
+    for (void* p : {(void*)lm.loop_step, (void*)lm.d_proj, (void*)lm.d_x0, (void*)lm.d_moe_y, (void*)lm.d_topk_w, lm.d_q, lm.d_plain, lm.d_lat,
                     lm.d_ff, lm.d_xx, lm.d_moe_x, (void*)lm.d_topk_ids, (void*)lm.d_offsets, (void*)lm.d_f2n, (void*)lm.d_en2f}) {
         if (p) {
             (void)hipFree(p);
@@ -585,8 +585,11 @@ static int wide_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts
         close.gate_bias = L.rg2_b;
     }
     if (s.mlp == TM_MLP_GATED) {
-        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_linear(L.gu, lm.d_h1, lm.ldw, lm.d_gu, lm.ldgu, M, kDenseScaleF32, 1.f, st)));
-        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_act_mul(lm.d_ff, lm.ldff, lm.elem, lm.d_gu, lm.ldgu, s.ff, M, s.ff, s.act, st)));
+        DenseCall c;  // act(gate) * up leaves the [gate | up] product's epilogue in the activation type
+        c.epi   = kDenseGatedAct;
+        c.act   = s.act;
+        c.n_out = s.ff;
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_call(L.gu, lm.d_h1, lm.ldw, lm.d_ff, lm.ldff, M, c, st)));
         TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_call(L.down, lm.d_ff, lm.ldff, lm.d_res, W, M, close, st)));
     }
     else if (s.mlp == TM_MLP_MOE) {
@@ -595,11 +598,13 @@ static int wide_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts
         TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_route(lm.d_offsets, lm.d_f2n, lm.d_en2f, lm.d_topk_ids, M, E, k, st)));
         TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_gather(lm.d_moe_x, lm.ldw, lm.d_h1, lm.ldw, lm.elem, lm.d_topk_w, lm.d_en2f, M, W, k, true, st)));
         DenseCall c;
-        c.epi         = kDenseScaleF32;
+        c.epi         = kDenseGatedAct;
+        c.act         = s.act;
+        c.n_out       = s.ff;
         c.count       = E;
         c.row_offsets = lm.d_offsets;
-        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_call(L.gu, lm.d_moe_x, lm.ldw, lm.d_gu, lm.ldgu, M * k, c, st)));
-        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_act_mul(lm.d_ff, lm.ldff, lm.elem, lm.d_gu, lm.ldgu, s.ff, M * k, s.ff, s.act, st)));
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_call(L.gu, lm.d_moe_x, lm.ldw, lm.d_ff, lm.ldff, M * k, c, st)));
+        c.epi = kDenseScaleF32;
         TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_call(L.down, lm.d_ff, lm.ldff, lm.d_moe_y, W, M * k, c, st)));
         TM_PROF(P_GEMM_DOWN, TM_TRY(launch_moe_combine_f32(lm.d_res, lm.d_moe_y, lm.d_topk_w, lm.d_en2f, s.resid_gate ? close.gate : nullptr, lm.ldproj,
                                                      close.gate_bias, M, W, k, false, st)));

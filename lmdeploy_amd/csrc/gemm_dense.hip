@@ -177,6 +177,24 @@ __global__ __launch_bounds__(WAVES * 64) void dense_skinny_bf16_kernel(const __b
         }
     }
     __syncthreads();
+    if (call.epi == kDenseGatedAct) {  // column tiles 2 j, 2 j + 1 of the image are the gate / up halves of output tile j
+        if constexpr (NT == 2) {
+            for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {
+                const int t = idx >> 8, l = (idx >> 2) & 63, i = idx & 3;
+                float     g = 0.f, u = 0.f;
+#pragma unroll
+                for (int wv = 0; wv < WAVES; wv += 4) {
+                    g += (red[wv][t * 2][l][i] + red[wv + 1][t * 2][l][i]) + (red[wv + 2][t * 2][l][i] + red[wv + 3][t * 2][l][i]);
+                    u += (red[wv][t * 2 + 1][l][i] + red[wv + 1][t * 2 + 1][l][i]) + (red[wv + 2][t * 2 + 1][l][i] + red[wv + 3][t * 2 + 1][l][i]);
+                }
+                const int m = t * 16 + (l >> 4) * 4 + i, n = (n0 >> 1) + (l & 15);
+                if (m < M && n < call.n_out) {
+                    ((__bf16*)y)[(size_t)(row_base + m) * ldy + col_base + n] = (__bf16)(act_apply(call.act, g) * u);
+                }
+            }
+        }
+        return;
+    }
     for (int idx = threadIdx.x; idx < MT * NT * 256; idx += WAVES * 64) {
         const int tj = idx >> 8, l = (idx >> 2) & 63, i = idx & 3;
         float     s  = 0.f;
@@ -270,6 +288,22 @@ __global__ __launch_bounds__(256) void dense_tiled_bf16_kernel(const __bf16* __r
         }
         __syncthreads();
     }
+    if (call.epi == kDenseGatedAct) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int m = m0 + wm + i * 16 + (lane >> 4) * 4 + q, n = ((n0 + wn) >> 1) + (j >> 1) * 16 + (lane & 15);
+                    if (m < M && n < call.n_out) {
+                        ((__bf16*)y)[(size_t)(row_base + m) * ldy + col_base + n] = (__bf16)(act_apply(call.act, acc[i][j][q]) * acc[i][j + 1][q]);
+                    }
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -330,6 +364,19 @@ __global__ __launch_bounds__(256) void dense_f32_kernel(const float* __restrict_
             }
         }
     }
+    if (call.epi == kDenseGatedAct) {  // a thread's columns are gate, gate, up, up of two outputs
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int m = m0 + tr + i, n = ((n0 + tc) >> 1) + j;
+                if (m < M && n < call.n_out) {
+                    ((float*)y)[(size_t)(row_base + m) * ldy + col_base + n] = act_apply(call.act, acc[i][j]) * acc[i][j + 2];
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -354,12 +401,16 @@ __host__ __device__ inline size_t dense_frag_index(int n, int k, int Kp)
 
 template<class T>
 __global__ void dense_place_kernel(T* __restrict__ dst, int Kp, int row0, int col0, const __bf16* __restrict__ src, int rows, int cols,
-                                   int transpose)
+                                   int transpose, int half)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < (size_t)rows * cols) {
         const int r = (int)(i / cols), c = (int)(i % cols);
-        const int n = row0 + (transpose ? c : r), k = col0 + (transpose ? r : c);  // transposed: the block's columns become output rows
+        int       n = row0 + (transpose ? c : r);  // transposed: the block's columns become output rows
+        const int k = col0 + (transpose ? r : c);
+        if (half) {
+            n = dense_pair_row(n, half - 1, sizeof(T) == 4);
+        }
         if constexpr (sizeof(T) == 2) {
             dst[dense_frag_index(n, k, Kp)] = (T)(float)src[i];
         }
@@ -384,19 +435,22 @@ int dense_weight_alloc(DenseWeight& d, int K, int N, int dtype, hipStream_t st, 
     return 0;
 }
 
-int dense_weight_place(DenseWeight& d, int row0, int col0, const void* src_bf16, int rows, int cols, hipStream_t st, int item, bool transpose)
+int dense_weight_place(DenseWeight& d, int row0, int col0, const void* src_bf16, int rows, int cols, hipStream_t st, int item, bool transpose,
+                       int half)
 {
-    TM_REQUIRE(d.w && row0 >= 0 && col0 >= 0 && item >= 0 && item < d.count, "dense weight: part outside the image");
-    TM_REQUIRE(row0 + (transpose ? cols : rows) <= d.N && col0 + (transpose ? rows : cols) <= d.K, "dense weight: part outside the image");
+    TM_REQUIRE(d.w && row0 >= 0 && col0 >= 0 && item >= 0 && item < d.count && half >= 0 && half <= 2, "dense weight: part outside the image");
+    TM_REQUIRE((half ? dense_pair_rows(row0 + (transpose ? cols : rows)) : row0 + (transpose ? cols : rows)) <= d.N
+                   && col0 + (transpose ? rows : cols) <= d.K,
+               "dense weight: part outside the image");
     const size_t n = (size_t)rows * cols, at = (size_t)item * d.Np * d.Kp;
     if (n == 0) {
         return 0;
     }
     if (d.dtype == kDenseF32) {
-        dense_place_kernel<float><<<(n + 255) / 256, 256, 0, st>>>((float*)d.w + at, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols, transpose);
+        dense_place_kernel<float><<<(n + 255) / 256, 256, 0, st>>>((float*)d.w + at, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols, transpose, half);
     }
     else {
-        dense_place_kernel<__bf16><<<(n + 255) / 256, 256, 0, st>>>((__bf16*)d.w + at, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols, transpose);
+        dense_place_kernel<__bf16><<<(n + 255) / 256, 256, 0, st>>>((__bf16*)d.w + at, d.Kp, row0, col0, (const __bf16*)src_bf16, rows, cols, transpose, half);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;
@@ -422,8 +476,10 @@ int launch_dense_call(const DenseWeight& d, const void* x, int ldx, void* y, int
 {
     const int epi = call.epi;
     TM_REQUIRE(d.w && x && y && M >= 0 && call.count >= 1 && call.count <= d.count, "dense linear: operands");
-    TM_REQUIRE(ldx >= d.Kp + (call.count - 1) * call.x_col_stride && ldy >= d.N + (call.count - 1) * call.y_col_stride, "dense linear: row lengths");
-    TM_REQUIRE(epi >= kDenseStore && epi <= kDenseResidGate, "dense linear: epilogue");
+    const int n_y = epi == kDenseGatedAct ? call.n_out : d.N;
+    TM_REQUIRE(ldx >= d.Kp + (call.count - 1) * call.x_col_stride && ldy >= n_y + (call.count - 1) * call.y_col_stride, "dense linear: row lengths");
+    TM_REQUIRE(epi >= kDenseStore && epi <= kDenseGatedAct, "dense linear: epilogue");
+    TM_REQUIRE(epi != kDenseGatedAct || (call.n_out >= 1 && dense_pair_rows(call.n_out) <= d.N), "dense linear: paired image");
     TM_REQUIRE(epi != kDenseBiasF32 || call.bias, "dense linear: bias");
     TM_REQUIRE(epi != kDenseResidGate || (call.gate && call.gate_bias && call.ldg >= d.N), "dense linear: gate");
     if (M == 0) {
@@ -440,7 +496,7 @@ int launch_dense_call(const DenseWeight& d, const void* x, int ldx, void* y, int
         TM_REQUIRE(ldx % 8 == 0 && call.x_col_stride % 8 == 0, "dense linear (bf16): rows and items must be 16-byte aligned");
         if (M <= 32) {
             // two column tiles per wave where that still leaves >= 512 workgroups (two per CU): wide outputs amortise the activation reads
-            const int nt     = d.N >= 512 * 32 ? 2 : 1;
+            const int nt     = (d.N >= 512 * 32 || epi == kDenseGatedAct) ? 2 : 1;  // (a gate / up pair is two adjacent tiles of one wave)
             const int wgs    = (d.N + 16 * nt - 1) / (16 * nt);
             const int chunk  = (nt == 1 ? 8 : 4) * 32;
             int       waves  = 4;  // ... and more waves per workgroup while the device holds fewer than 16 per CU and K has a chunk for each

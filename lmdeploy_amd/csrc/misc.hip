@@ -7,7 +7,6 @@
 //           QuantizeGroupwise / IntegralQuantizer (kernels/quantization.cu:384-440,515-676).
 #include "tm_common.h"
 #include "tm_kernels.h"
-#include "../../include/tm_mi355x.h"
 #include <map>
 #include <mutex>
 
@@ -343,47 +342,6 @@ int launch_f32_to_f16_rows(half_t* out, int ld, const float* in, int n, int V, h
 }
 
 // ---- fp32 stream helpers of the layer-list family ------------------------------------------------------------------------------------
-__device__ __forceinline__ float act_apply(int act, float z)
-{
-    if (act == TM_ACT_GELU_TANH) {
-        return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-    }
-    if (act == TM_ACT_SILU) {
-        return z / (1.f + expf(-z));
-    }
-    const float r = fmaxf(z, 0.f);
-    return r * r;
-}
-
-// out[m][i] = act(gu[m][i]) * gu[m][up_col + i]: the gated feed-forward's activation between its two products
-template<class T>
-__global__ void act_mul_kernel(T* __restrict__ out, int ldo, const float* __restrict__ gu, int ld, int up_col, int n, int act, size_t total)
-{
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < total) {
-        const size_t m = i / n;
-        const int    c = (int)(i % n);
-        out[m * ldo + c] = (T)(act_apply(act, gu[m * ld + c]) * gu[m * ld + up_col + c]);
-    }
-}
-
-int launch_act_mul(void* out, int ldo, int out_elem_bytes, const float* gu, int ld, int up_col, int M, int n, int act, hipStream_t st)
-{
-    TM_REQUIRE(out && gu && ldo >= n && ld >= up_col + n && (out_elem_bytes == 2 || out_elem_bytes == 4), "act_mul: operands");
-    const size_t total = (size_t)M * n;
-    if (total == 0) {
-        return 0;
-    }
-    if (out_elem_bytes == 2) {
-        act_mul_kernel<__bf16><<<(total + 255) / 256, 256, 0, st>>>((__bf16*)out, ldo, gu, ld, up_col, n, act, total);
-    }
-    else {
-        act_mul_kernel<float><<<(total + 255) / 256, 256, 0, st>>>((float*)out, ldo, gu, ld, up_col, n, act, total);
-    }
-    TM_HIP_CHECK(hipGetLastError());
-    return 0;
-}
-
 // out[m] = [a[m] | b[m]] in the activation type: two fp32 streams side by side as the operand of one product
 template<class T>
 __global__ void concat2_kernel(T* __restrict__ out, int ldo, const float* __restrict__ a, const float* __restrict__ b, int H, size_t total)

@@ -341,8 +341,32 @@ inline uint64_t* gemm_trace_for(size_t workgroups, const char* tag = "", int gx 
 // ---- gemm_dense.hip: unquantised linears, W stored [N][K]; bf16 on the matrix cores or true fp32 ------------------------------
 enum { kDenseBf16 = 0, kDenseF32 = 1 };
 // epilogues: y = acc (activation type) | y = relu(acc)^2 | y_f32 += alpha * acc (residual stream) | y_f32 = alpha * acc |
-// y_f32 = acc + bias[n] | y_f32 += sigmoid(gate[m][n] + gate_bias[n]) * acc (gated residual sum)
-enum { kDenseStore = 0, kDenseRelu2 = 1, kDenseResidAdd = 2, kDenseScaleF32 = 3, kDenseBiasF32 = 4, kDenseResidGate = 5 };
+// y_f32 = acc + bias[n] | y_f32 += sigmoid(gate[m][n] + gate_bias[n]) * acc (gated residual sum) |
+// y[m][n] = act(acc_gate[m][n]) * acc_up[m][n] (activation type; the image holds the [gate | up] pair of a gated feed-forward interleaved
+// so that both accumulators of an output element live in one thread: dense_weight_place with half = 1 / 2)
+enum { kDenseStore = 0, kDenseRelu2 = 1, kDenseResidAdd = 2, kDenseScaleF32 = 3, kDenseBiasF32 = 4, kDenseResidGate = 5, kDenseGatedAct = 6 };
+enum { kActRelu2 = 0, kActGeluTanh = 1, kActSilu = 2 };  // (= TM_ACT_*)
+__device__ __forceinline__ float act_apply(int act, float z)
+{
+    if (act == kActGeluTanh) {
+        return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    }
+    if (act == kActSilu) {
+        return z / (1.f + expf(-z));
+    }
+    const float r = fmaxf(z, 0.f);
+    return r * r;
+}
+// image rows of a paired [gate | up] weight: output n's gate row (half 0) and up row (half 1).  bf16: 16-column tiles alternate (a wave's two
+// adjacent MFMA tiles hold the pair in the same lane and register); fp32: column pairs alternate (a thread's four columns are g g u u)
+__host__ __device__ inline int dense_pair_row(int n, int half, bool f32)
+{
+    return f32 ? (n >> 1) * 4 + half * 2 + (n & 1) : (n >> 4) * 32 + half * 16 + (n & 15);
+}
+inline int dense_pair_rows(int n_out)  // rows of a paired image for n_out outputs (either format fits)
+{
+    return (n_out + 15) / 16 * 32;
+}
 struct DenseWeight {
     int    K = 0, N = 0, Kp = 0, Np = 0;  // Kp = K rounded up to 32, Np = N rounded up to 128: zero-padded image [Np][Kp]
     int    dtype = kDenseBf16;
@@ -358,6 +382,7 @@ struct DenseCall {
     const float* gate  = nullptr;       // kDenseResidGate: gate logits [M][ldg] and their bias [N]
     const float* gate_bias = nullptr;
     int          ldg   = 0;
+    int          act = kActRelu2, n_out = 0;  // kDenseGatedAct: the activation and the number of outputs (the image has 2 rows per output)
     int          count = 1;             // items; item g uses image g, x column g * x_col_stride, y column g * y_col_stride ...
     int          x_col_stride = 0, y_col_stride = 0;
     const int*   row_offsets = nullptr; // ... and, when set, the rows [row_offsets[g], row_offsets[g + 1]) of x and y (device, [count + 1])
@@ -367,7 +392,7 @@ int  dense_weight_alloc(DenseWeight& d, int K, int N, int dtype, hipStream_t st,
 // rows x cols bf16 block (checkpoint orientation [out][in]) -> image rows [row0, row0 + rows), columns [col0, col0 + cols):
 // concatenation along N fuses projections of one input, along K projections that are summed.  transpose: the block is [in][out]
 int  dense_weight_place(DenseWeight& d, int row0, int col0, const void* src_bf16, int rows, int cols, hipStream_t st, int item = 0,
-                        bool transpose = false);
+                        bool transpose = false, int half = 0 /* 1: gate rows, 2: up rows of a paired image (row0 counts outputs) */);
 void dense_weight_free(DenseWeight& d);
 int  launch_dense_call(const DenseWeight& d, const void* x, int ldx, void* y, int ldy, int M, DenseCall call, hipStream_t st);
 // x [M][ldx] (ldx >= Kp, pad columns finite), y [M][ldy]; x / y element type = the weight's dtype unless the epilogue says fp32
@@ -435,8 +460,6 @@ int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col,
 int launch_latent_prep(const float* proj, int ld, int q_col, int dkv_col, void* q_plain, int ldp, int plain_stride, void* q_full, int ldq,
                        const float* c_norm_w, const float* inv_freq, int D, int R, int C, float eps, const GeneralAttnParams& layout,
                        hipStream_t st);
-// out[m][i] = act(gu[m][i]) * gu[m][up_col + i] (act: TM_ACT_*), out bf16 | fp32
-int launch_act_mul(void* out, int ldo, int out_elem_bytes, const float* gu, int ld, int up_col, int M, int n, int act, hipStream_t st);
 // out[m] = [a[m] | b[m]] (a, b fp32 [M][H]) in bf16 | fp32
 int launch_concat2(void* out, int ldo, int out_elem_bytes, const float* a, const float* b, int M, int H, hipStream_t st);
 // mixture of experts on the fp32 stream: sigmoid router top-k from fp32 logits; gather (optionally scaled) rows in expert order; gated sum

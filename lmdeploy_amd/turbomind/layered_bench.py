@@ -141,10 +141,12 @@ def _decode_bytes(s, batch, ctx, fokonex: bool):
     return b
 
 
-def run(steps: int, warmup: int, batch: int, prompt_len: int, sizes=None, design: str = 'fokonex') -> dict:
+def run(steps: int, warmup: int, batch: int, prompt_len: int, sizes=None, design: str = 'fokonex', only_first: bool = False) -> dict:
     res = {}
     pair = (('fokonex_bf16', _fokonex_engine), ('llama_f16', _llama_engine)) if design == 'fokonex' else \
         (('bedenex_bf16', _bedenex_engine), ('fokonex_bf16', _fokonex_engine))
+    if only_first:
+        pair = pair[:1]
     for name in (sizes or SIZES):
         s = SIZES[name]
         session_len = prompt_len + steps + warmup + 64
@@ -159,6 +161,9 @@ def run(steps: int, warmup: int, batch: int, prompt_len: int, sizes=None, design
                                                  for k in need if m['decode_categories_ms'].get(k)}
             eng.close()
             row[kind] = m
+        if only_first:
+            res[name] = row
+            continue
         f, l = row[pair[0][0]], row[pair[1][0]]
         if design != 'fokonex':   # how much farther from its roofline each category of the new design runs than the like one beside it
             fa, fb = f['decode_hbm_roofline_fraction'], l['decode_hbm_roofline_fraction']
