@@ -683,10 +683,11 @@ bool general_attention_tiles_ok(const GeneralAttnParams& p)
 }
 
 // row tiles per wave of the prefill kernel (64 * RT query rows per workgroup): as many as the register file holds without scratch --
-// every key / value fragment a wave loads then serves 16 * RT query rows
+// every key / value fragment a wave loads then serves 16 * RT query rows.  (Key sizes up to 256 with value sizes up to 192 -- the latent
+// space of latent attention -- still hold two: 256 VGPRs + 184 AGPRs.)
 constexpr int tile_rt(int ds, int vt)
 {
-    return (ds <= 4 && vt <= 8) ? 4 : ((ds <= 4 || vt <= 8) ? 2 : 1);
+    return (ds <= 4 && vt <= 8) ? 4 : ((ds <= 4 || vt <= 8 || (ds <= 8 && vt <= 12)) ? 2 : 1);
 }
 
 // value sizes are served by the next even tile count (the kernels test channel < vdim), key sizes by 1, 2, 3, 4, 6 or 8 steps

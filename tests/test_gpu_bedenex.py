@@ -107,6 +107,7 @@ ATT = {
     'tiny_chunks': dict(heads=3, kv_heads=3, dim=72, vdim=136, scale=0.1, chunk=7, r1=None),
     'one_chunk': dict(heads=2, kv_heads=1, dim=20, vdim=12, scale=0.2, chunk=1000, r1=[1.5, 0.7], r2=[0.4, 0.1]),
     'no_chunk': dict(heads=16, kv_heads=1, dim=48, vdim=32, scale=0.15, chunk=0, r1=[0.1 * i for i in range(16)], r2=[0.2] * 16),
+    'latent_sized': dict(heads=5, kv_heads=1, dim=256, vdim=192, scale=0.06, chunk=0, r1=None),     # one shared key head, the largest tile kernel
 }
 
 
