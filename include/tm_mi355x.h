@@ -521,8 +521,8 @@ enum { TM_DTYPE_BF16 = 0, TM_DTYPE_F32 = 1 };
  *                inside its own chunk, floor(i / chunk) = floor(j / chunk); out_gate: head h's output *= sigmoid(g h)[h] ("mix.g" [heads][width])
  *   TM_MIXER_LATENT: per token one latent vector c = norm(dkv h [0, kv_rank)) * "mix.dkv.norm" and one rotated key part
  *                rot(dkv h [kv_rank, kv_rank + rot_dim)) shared by all heads are cached; head a: key = [uk_a c | rotated part], value = uv_a c,
- *                query = [q_a h [0, dim) | rot(q_a h [dim, dim + rot_dim))]; rotation pairs channel i with i + rot_dim / 2, angle =
- *                position * rot_base^(-2 i / rot_dim); causal; sink as above.  kv_heads = 1.  Slots "mix.q" [heads (dim + rot_dim)][width],
+ *                query = [q_a h [0, dim) | rot(q_a h [dim, dim + rot_dim))]; rotation of the first rot_dims channels (0: all rot_dim) pairs
+ *                channel i with i + rot_dims / 2, angle = position * rot_base^(-2 i / rot_dims); causal; sink as above.  kv_heads = 1.  Slots "mix.q" [heads (dim + rot_dim)][width],
  *                "mix.dkv" [kv_rank + rot_dim][width], "mix.dkv.norm", "mix.uk" [heads dim][kv_rank], "mix.uv" [heads vdim][kv_rank], "mix.o"
  *   TM_MLP_GATED: down(act(gate h) * (up h)) ("mlp.gate", "mlp.up", "mlp.down"); act TM_ACT_GELU_TANH | TM_ACT_SILU | TM_ACT_RELU2
  *   TM_MLP_MOE:  `experts` gated feed-forwards of size ff ("mlp.e<j>.gate|up|down"), router scores sigmoid("mlp.router" h) in fp32, the
@@ -539,6 +539,7 @@ typedef struct tm_layer_spec {
     int   kv_rank, rot_dim;
     float rot_base;
     int   experts, top;
+    int   rot_dims; /* how many of the rot_dim channels turn (the first ones; the rest pass unchanged); 0: all */
 } tm_layer_spec;
 typedef struct tm_layered_config {
     int                  width, vocab, n_layers;

@@ -73,7 +73,7 @@ class LayerSpec(C.Structure):
                 ('scale', c_float), ('softcap', c_float), ('qtemp_coef', c_float), ('qtemp_every', c_float), ('sink', c_int),
                 ('mlp', c_int), ('ff', c_int), ('act', c_int), ('one_norm', c_int), ('resid_gate', c_int), ('loop_pass', c_int),
                 ('qk_unit_norm', c_int), ('v_unit_norm', c_int), ('dist_bias', c_int), ('out_gate', c_int), ('chunk', c_int),
-                ('kv_rank', c_int), ('rot_dim', c_int), ('rot_base', c_float), ('experts', c_int), ('top', c_int)]
+                ('kv_rank', c_int), ('rot_dim', c_int), ('rot_base', c_float), ('experts', c_int), ('top', c_int), ('rot_dims', c_int)]
 
 
 class LayeredConfig(C.Structure):

@@ -110,12 +110,15 @@ static int process_wide_layer(tm_engine* e, int i, LmLayer& L, int dt)
             TM_TRY(place(e, L.uk, 0, 0, lname(i, "mix.uk"), s.dim, C, (size_t)h * s.dim, h, true));
             TM_TRY(place(e, L.uv, 0, 0, lname(i, "mix.uv"), s.vdim, C, (size_t)h * s.vdim, h, false));
         }
-        std::vector<float> f(R / 2);
-        for (int j = 0; j < R / 2; ++j) {
-            f[j] = (float)std::pow((double)s.rot_base, -2.0 * j / R);
+        const int          rd = s.rot_dims > 0 ? s.rot_dims : R;
+        std::vector<float> f(rd / 2);
+        for (int j = 0; j < rd / 2; ++j) {
+            f[j] = (float)std::pow((double)s.rot_base, -2.0 * j / rd);
         }
-        TM_TRY(dmalloc(&L.inv_freq, (size_t)std::max(1, R / 2)));
-        TM_HIP_CHECK(hipMemcpyAsync(L.inv_freq, f.data(), f.size() * 4, hipMemcpyHostToDevice, e->stream));
+        TM_TRY(dmalloc(&L.inv_freq, (size_t)std::max(1, rd / 2)));
+        if (!f.empty()) {
+            TM_HIP_CHECK(hipMemcpyAsync(L.inv_freq, f.data(), f.size() * 4, hipMemcpyHostToDevice, e->stream));
+        }
         TM_HIP_CHECK(hipStreamSynchronize(e->stream));
     }
     else {
@@ -540,7 +543,7 @@ static int wide_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts
         if (latent) {
             TM_PROF(P_KV_STORE, TM_TRY(launch_latent_prep(proj, lm.ldproj, 0, L.c_k, (char*)lm.d_plain + (size_t)P.row0 * lm.ldplain * lm.elem, lm.ldplain,
                                                           L.plain_stride, (void*)p.q, lm.ldq, L.c_norm, L.inv_freq, s.dim, s.rot_dim, s.kv_rank,
-                                                          m.norm_eps, p, st)));
+                                                          s.rot_dims > 0 ? s.rot_dims : s.rot_dim, m.norm_eps, p, st)));
         }
         else {
             TM_PROF(P_KV_STORE, TM_TRY(launch_attn_prep(proj, lm.ldproj, 0, L.c_k, L.c_v, (void*)p.q, lm.ldq, s.qk_unit_norm != 0, s.v_unit_norm != 0,
@@ -741,6 +744,7 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
                        at + ": feed-forward");
             TM_REQUIRE(s.mlp != TM_MLP_MOE || (s.experts >= 1 && s.experts <= 1024 && s.top >= 1 && s.top <= s.experts), at + ": 1 <= top <= experts <= 1024");
             if (s.mixer == TM_MIXER_LATENT) {
+                TM_REQUIRE(s.rot_dims >= 0 && s.rot_dims <= s.rot_dim && s.rot_dims % 2 == 0, at + ": rot_dims even, <= rot_dim");
                 TM_REQUIRE(s.kv_heads == 1 && s.kv_rank >= 1 && s.rot_dim >= 0 && s.rot_dim % 2 == 0 && s.kv_rank + s.rot_dim <= 1024 && s.rot_base > 0.f,
                            at + ": latent attention: kv_heads 1, kv_rank >= 1, rot_dim even, kv_rank + rot_dim <= 1024");
                 TM_REQUIRE(!s.qk_unit_norm && !s.v_unit_norm && !s.out_gate, at + ": latent attention has no per-head unit norms and no output gate");

@@ -464,15 +464,15 @@ int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col,
 // proj [rows][ld]: queries at q_col, head h as [D unrotated | R rotated]; at dkv_col the C latent channels, then the R rotated ones.
 //   q_plain [rows][ldp], head h at h * plain_stride : unrotated query parts (input of the key-expansion product)
 //   q_full  [rows][ldq], head h at h * (C + R)      : the rotated part goes to [C, C + R) (the product fills [0, C))
-// Rotation pairs channel i with i + R / 2; angle = position * inv_freq[i], fp32.
+// Rotation turns the first `rd` of the R channels: channel i pairs with i + rd / 2, angle = position * inv_freq[i], fp32; the rest pass.
 template<class T>
 __global__ __launch_bounds__(256) void latent_prep_kernel(const float* __restrict__ proj, int ld, int q_col, int dkv_col, T* __restrict__ q_plain,
                                                           int ldp, int plain_stride, T* __restrict__ q_full, int ldq,
                                                           const float* __restrict__ c_norm_w, const float* __restrict__ inv_freq, int D, int R, int C,
-                                                          float eps, GeneralAttnParams p)
+                                                          int rd, float eps, GeneralAttnParams p)
 {
     __shared__ float red[4];
-    const int    t = blockIdx.x, H = p.q_heads, half = R / 2;
+    const int    t = blockIdx.x, H = p.q_heads, half = rd / 2, still = R - rd;
     const int    s = p.row_seq[t], pos = p.row_pos[t], ti = pos % p.block_len;
     const float* x = proj + (size_t)t * ld;
     for (int i = threadIdx.x; i < H * D; i += 256) {
@@ -487,6 +487,10 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const float* __restric
         T* q = q_full + (size_t)t * ldq + (size_t)h * (C + R) + C;
         q[f]        = (T)(u * cs - v * sn);
         q[f + half] = (T)(v * cs + u * sn);
+    }
+    for (int i = threadIdx.x; i < H * still; i += 256) {  // channels of the rotated part that do not turn
+        const int h = i / still, f = rd + i % still;
+        q_full[(size_t)t * ldq + (size_t)h * (C + R) + C + f] = (T)x[q_col + h * (D + R) + D + f];
     }
     char* base = (char*)p.block_ptrs[(size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride + pos / p.block_len] + p.layer_offset;
     T*    k    = (T*)base + (size_t)ti * (C + R);
@@ -513,23 +517,27 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const float* __restric
         k[C + f]        = (T)(u * cs - v * sn);
         k[C + f + half] = (T)(v * cs + u * sn);
     }
+    for (int f = rd + threadIdx.x; f < R; f += 256) {
+        k[C + f] = (T)x[dkv_col + C + f];
+    }
 }
 
 int launch_latent_prep(const float* proj, int ld, int q_col, int dkv_col, void* q_plain, int ldp, int plain_stride, void* q_full, int ldq,
-                       const float* c_norm_w, const float* inv_freq, int D, int R, int C, float eps, const GeneralAttnParams& p, hipStream_t st)
+                       const float* c_norm_w, const float* inv_freq, int D, int R, int C, int rd, float eps, const GeneralAttnParams& p,
+                       hipStream_t st)
 {
     TM_REQUIRE(proj && q_plain && q_full && c_norm_w && inv_freq && p.row_seq && p.row_pos && p.block_ptrs, "latent_prep: operands");
-    TM_REQUIRE(R % 2 == 0 && p.kv_heads == 1 && p.dim == C + R && p.vdim == C && plain_stride >= D, "latent_prep: sizes");
+    TM_REQUIRE(rd % 2 == 0 && rd >= 0 && rd <= R && p.kv_heads == 1 && p.dim == C + R && p.vdim == C && plain_stride >= D, "latent_prep: sizes");
     if (p.rows == 0) {
         return 0;
     }
     if (p.elem_bytes == 2) {
         latent_prep_kernel<__bf16><<<p.rows, 256, 0, st>>>(proj, ld, q_col, dkv_col, (__bf16*)q_plain, ldp, plain_stride, (__bf16*)q_full, ldq, c_norm_w,
-                                                           inv_freq, D, R, C, eps, p);
+                                                           inv_freq, D, R, C, rd, eps, p);
     }
     else {
         latent_prep_kernel<float><<<p.rows, 256, 0, st>>>(proj, ld, q_col, dkv_col, (float*)q_plain, ldp, plain_stride, (float*)q_full, ldq, c_norm_w,
-                                                          inv_freq, D, R, C, eps, p);
+                                                          inv_freq, D, R, C, rd, eps, p);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;

@@ -458,8 +458,8 @@ int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col,
 // latent attention (layout: one key head, dim = C + R, vdim = C): normed latent vector + rotated shared key part -> cache; unrotated query
 // parts -> q_plain (head h at h * plain_stride), rotated query parts -> q_full[h * (C + R) + C ...]
 int launch_latent_prep(const float* proj, int ld, int q_col, int dkv_col, void* q_plain, int ldp, int plain_stride, void* q_full, int ldq,
-                       const float* c_norm_w, const float* inv_freq, int D, int R, int C, float eps, const GeneralAttnParams& layout,
-                       hipStream_t st);
+                       const float* c_norm_w, const float* inv_freq, int D, int R, int C, int rot_dims, float eps,
+                       const GeneralAttnParams& layout, hipStream_t st);
 // out[m] = [a[m] | b[m]] (a, b fp32 [M][H]) in bf16 | fp32
 int launch_concat2(void* out, int ldo, int out_elem_bytes, const float* a, const float* b, int M, int H, hipStream_t st);
 // mixture of experts on the fp32 stream: sigmoid router top-k from fp32 logits; gather (optionally scaled) rows in expert order; gated sum

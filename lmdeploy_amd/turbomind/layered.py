@@ -60,6 +60,7 @@ class LayerSpec:
     rot_base: float = 10000.0
     experts: int = 0
     top: int = 0
+    rot_dims: int = 0             # how many channels of the rotated part turn (0: all of them)
 
 
 @dataclass
@@ -82,7 +83,7 @@ class LayeredConfig:
         arr = (_ffi.LayerSpec * len(self.layers))(*[
             _ffi.LayerSpec(s.mixer, s.weights_of, s.heads, s.kv_heads, s.dim, s.vdim, s.scale, s.softcap, s.qtemp_coef, s.qtemp_every,
                            int(s.sink), s.mlp, s.ff, s.act, int(s.one_norm), int(s.resid_gate), s.loop_pass, int(s.qk_unit_norm),
-                           int(s.v_unit_norm), int(s.dist_bias), int(s.out_gate), s.chunk, s.kv_rank, s.rot_dim, s.rot_base, s.experts, s.top)
+                           int(s.v_unit_norm), int(s.dist_bias), int(s.out_gate), s.chunk, s.kv_rank, s.rot_dim, s.rot_base, s.experts, s.top, s.rot_dims)
             for s in self.layers])
         return _ffi.LayeredConfig(self.width, self.vocab, len(self.layers), arr, self.norm_eps, self.norm_offset, self.residual_mult,
                                   self.logit_scale, DTYPES[dtype], self.loop_times), arr
@@ -151,8 +152,9 @@ def _bedenex_layer(i: int, L: dict) -> LayerSpec:
     elif L['type'] == 'latent_attention':
         s.mixer, s.kv_heads, s.sink = MIXER_LATENT, 1, True
         s.kv_rank, s.rot_dim, s.rot_base = int(m['kv_rank']), int(m['rot_dim']), float(m['rot']['base'])
-        if int(m['rot'].get('dims', s.rot_dim)) != s.rot_dim:
-            raise NotImplementedError(f'layer {i}: the whole rotated part turns (rot.dims == rot_dim)')
+        s.rot_dims = int(m['rot'].get('dims', s.rot_dim))
+        if not 0 <= s.rot_dims <= s.rot_dim or s.rot_dims % 2:
+            raise ValueError(f'layer {i}: rot.dims must be even and at most rot_dim')
     else:
         raise NotImplementedError(f'layer {i}: mixer {L["type"]!r}')
     if mlp is None:

@@ -34,8 +34,11 @@ def rms_norm(x, w, eps):
     return unit_rms(x, eps) * w
 
 
-def rotate_half(x, pos, base):
-    """x [T, ..., d]: channel i pairs with i + d/2; the pair turns by the angle pos * base^(-2i/d)"""
+def rotate_half(x, pos, base, dims=None):
+    """x [T, ..., n]: of the first d = dims channels (all when None) channel i pairs with i + d/2 and the pair turns by the angle
+    pos * base^(-2i/d); channels from d on pass unchanged"""
+    if dims is not None and dims < x.shape[-1]:
+        return np.concatenate([rotate_half(x[..., :dims], pos, base), x[..., dims:]], axis=-1) if dims else x
     d = x.shape[-1]
     half = d // 2
     freq = base ** (-2.0 * np.arange(half) / d)
@@ -92,10 +95,11 @@ def latent_attention(h, t, m, eps):
     H, D, R, V, C = m['heads'], m['dim'], m['rot_dim'], m['vdim'], m['kv_rank']
     pos = np.arange(T)
     q = (h @ t['q'].T).reshape(T, H, D + R)
-    q_plain, q_rot = q[..., :D], rotate_half(q[..., D:], pos, m['rot']['base'])
+    dims = m['rot'].get('dims', R)
+    q_plain, q_rot = q[..., :D], rotate_half(q[..., D:], pos, m['rot']['base'], dims)
     dkv = h @ t['dkv'].T
     c = rms_norm(dkv[:, :C], t['dkv.norm'], eps)
-    k_rot = rotate_half(dkv[:, C:], pos, m['rot']['base'])  # [T, R]
+    k_rot = rotate_half(dkv[:, C:], pos, m['rot']['base'], dims)  # [T, R]
     k_plain = (c @ t['uk'].T).reshape(T, H, D)
     v = (c @ t['uv'].T).reshape(T, H, V)
     i, j = np.arange(T)[:, None], np.arange(T)[None, :]
@@ -207,10 +211,10 @@ def attention_layer(heads, kv_heads, dim, vdim, scale, chunk, mlp=None):
     return {'type': 'attention', 'mixer': m, 'mlp': mlp}
 
 
-def latent_layer(heads, dim, rot_dim, vdim, kv_rank, scale, base=10000.0, mlp=None):
+def latent_layer(heads, dim, rot_dim, vdim, kv_rank, scale, base=10000.0, mlp=None, dims=None):
     return {'type': 'latent_attention', 'mlp': mlp,
             'mixer': {'heads': heads, 'dim': dim, 'rot_dim': rot_dim, 'vdim': vdim, 'kv_rank': kv_rank, 'scale': scale,
-                      'rot': {'base': base, 'dims': rot_dim}}}
+                      'rot': {'base': base, 'dims': rot_dim if dims is None else dims}}}
 
 
 def dense(ff):
