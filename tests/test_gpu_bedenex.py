@@ -224,7 +224,7 @@ ALONE = {
     'attention': lambda: bo.make_config(64, 97, [bo.attention_layer(4, 1, 16, 32, 0.5, 33)]),
     'attention_plain_causal': lambda: bo.make_config(48, 97, [bo.attention_layer(2, 2, 40, 8, 0.2, 0)]),
     'latent': lambda: bo.make_config(64, 97, [bo.latent_layer(4, 24, 8, 16, 48, 0.3)]),
-    'latent_part_turns': lambda: bo.make_config(64, 97, [bo.latent_layer(3, 8, 24, 16, 40, 0.3, 300.0, dims=10)]),
+    'latent_part_turns': lambda: bo.make_config(64, 97, [bo.latent_layer(3, 8, 24, 16, 42, 0.3, 300.0, dims=10)]),      # latent size off the 8 grid
     'latent_wide': lambda: bo.make_config(40, 97, [bo.latent_layer(2, 12, 36, 20, 280, 0.1, 77.0)]),       # key size 316: beyond the tile kernels
     'gated_gelu': lambda: bo.make_config(64, 97, [bo.attention_layer(2, 1, 8, 8, 0.3, 16, bo.dense(100))]),
     'experts_top1': lambda: bo.make_config(64, 97, [bo.attention_layer(2, 1, 8, 8, 0.3, 16, bo.moe(3, 1, 24))]),
