@@ -97,7 +97,6 @@ static int process_wide_layer(tm_engine* e, int i, LmLayer& L, int dt)
 {
     const tm_layer_spec& s = L.spec;
     const int            W = e->lm->cfg.width, H = s.heads;
-    int                  n = L.n_q;
     TM_TRY(dense_weight_alloc(L.qkv, W, L.c_router + (s.mlp == TM_MLP_MOE ? s.experts : 0), dt, e->stream));
     TM_TRY(place(e, L.qkv, 0, 0, lname(i, "mix.q"), L.n_q, W));
     if (s.mixer == TM_MIXER_LATENT) {
@@ -128,7 +127,6 @@ static int process_wide_layer(tm_engine* e, int i, LmLayer& L, int dt)
             TM_TRY(place(e, L.qkv, L.c_g, 0, lname(i, "mix.g"), H, W));
         }
     }
-    (void)n;
     if (s.dist_bias) {
         TM_TRY(to_f32(e, lname(i, "mix.r1"), H, &L.r1));
         TM_TRY(to_f32(e, lname(i, "mix.r2"), H, &L.r2));
